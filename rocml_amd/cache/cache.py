@@ -30,7 +30,7 @@ import numpy as np
 import torch
 
 from ..errors import CacheFullError, MemoryBudgetError, RocmlError
-from ..parts.base import KVCacheRequest, StateRequest
+from ..parts.base import KVCacheRequest, LatentCacheRequest, StateRequest
 
 PAGE_SIZE = 64
 
@@ -124,13 +124,25 @@ class PagedGroup(CacheGroup):
     the group give pages back once no later query can see them.  Storage is the subclass's."""
     paged = True
 
-    def __init__(self, name: str, request, n_lines: int, n_pages: int, page_size: int, window: Optional[int]):
+    def __init__(self, name: str, request, n_lines: int, n_pages: int, page_size: int, window: Optional[int],
+                 chunk: Optional[int] = None):
         super().__init__(name, request, n_lines)
         self.n_pages = n_pages
         self.page_size = page_size
+        # ``window``: a query sees the last so many positions.  ``chunk``: a query sees its own block
+        # of so many positions, counted from 0.  Either way the group gives back the pages that lie
+        # wholly before what the next query can see; ``span`` is the most positions that can be.
         self.window = window
+        self.chunk = chunk
+        self.span = window if window is not None else chunk
         self._free = list(range(n_pages - 1, -1, -1))
         self._pages: Dict[int, List[int]] = {}   # slot -> logical page -> pool page, -1 once released
+
+    @staticmethod
+    def span_of(request) -> Optional[int]:
+        """The most positions a query of this request looks back over (None: all)."""
+        window, chunk = getattr(request, "window", None), getattr(request, "chunk", None)
+        return window if window is not None else chunk
 
     @staticmethod
     def pool_pages(window: Optional[int], geo: Geometry) -> int:
@@ -180,13 +192,20 @@ class PagedGroup(CacheGroup):
     def committed(self, slot: int, length: int) -> None:
         self.trim(slot, length)
 
+    def first_visible(self, length: int) -> int:
+        """The first position that a query at position ``length`` or later can still see."""
+        if self.window is not None:
+            return max(0, length - self.window + 1)
+        if self.chunk is not None:
+            return length - length % self.chunk
+        return 0
+
     def trim(self, slot: int, length: int) -> None:
-        """After a sequence reached ``length``: a group with a window releases the pages
+        """After a sequence reached ``length``: a group with a window or blocks releases the pages
         whose positions no query at ``length`` or later can see."""
-        w = self.window
-        if w is None:
+        if self.span is None:
             return
-        first_needed = max(0, length - w + 1) // self.page_size
+        first_needed = self.first_visible(length) // self.page_size
         table = self._pages[slot]
         for i in range(min(first_needed, len(table))):
             if table[i] >= 0:
@@ -217,19 +236,22 @@ class KVGroup(PagedGroup):
     """Paged keys and values of the cache lines that share one ``KVCacheRequest``."""
 
     def __init__(self, name: str, request: KVCacheRequest, n_lines: int, geo: Geometry):
-        super().__init__(name, request, n_lines, self.pool_pages(request.window, geo), geo.page_size, request.window)
+        super().__init__(name, request, n_lines, self.pool_pages(self.span_of(request), geo), geo.page_size,
+                         request.window, getattr(request, "chunk", None))
         # Values are transposed inside a page, which is the order the attention kernels
         # multiply them in.  Zeroed once: rows beyond a sequence's length are never counted,
         # but they are multiplied by a zero weight and so must stay finite.
         h, d = request.n_kv_heads, request.head_dim
+        dv = d if getattr(request, "v_head_dim", None) is None else request.v_head_dim
         self.k = torch.zeros((n_lines, self.n_pages, h, self.page_size, d), dtype=geo.dtype, device=geo.device)
-        self.v = torch.zeros((n_lines, self.n_pages, h, d, self.page_size), dtype=geo.dtype, device=geo.device)
+        self.v = torch.zeros((n_lines, self.n_pages, h, dv, self.page_size), dtype=geo.dtype, device=geo.device)
 
     @staticmethod
     def planned_bytes(request: KVCacheRequest, n_lines: int, geo: Geometry) -> int:
         size = torch.empty((), dtype=geo.dtype).element_size()
-        return (2 * n_lines * PagedGroup.pool_pages(request.window, geo) * geo.page_size
-                * request.n_kv_heads * request.head_dim * size)
+        dv = request.head_dim if getattr(request, "v_head_dim", None) is None else request.v_head_dim
+        return (n_lines * PagedGroup.pool_pages(PagedGroup.span_of(request), geo) * geo.page_size
+                * request.n_kv_heads * (request.head_dim + dv) * size)
 
     def view(self, line: int, step) -> "CacheLineView":
         return CacheLineView(group=self, line=line, k=self.k[line], v=self.v[line],
@@ -237,7 +259,30 @@ class KVGroup(PagedGroup):
 
     def bytes_per_token(self) -> int:
         r = self.request
-        return 2 * self.n_lines * r.n_kv_heads * r.head_dim * self.k.element_size()
+        return self.n_lines * r.n_kv_heads * (r.head_dim + self.v.shape[3]) * self.k.element_size()
+
+
+class LatentGroup(PagedGroup):
+    """Paged rows of the cache lines that share one ``LatentCacheRequest``: one row of ``width``
+    numbers per position, ``[line, page, page_size, width]``, in the model's compute type.  A
+    mixer sees its line as ``view.k``; there is nothing per head and no separate values."""
+
+    def __init__(self, name: str, request: LatentCacheRequest, n_lines: int, geo: Geometry):
+        super().__init__(name, request, n_lines, self.pool_pages(self.span_of(request), geo), geo.page_size,
+                         request.window, request.chunk)
+        # zeroed once, for the same reason as keys and values
+        self.k = torch.zeros((n_lines, self.n_pages, self.page_size, request.width), dtype=geo.dtype, device=geo.device)
+
+    @staticmethod
+    def planned_bytes(request: LatentCacheRequest, n_lines: int, geo: Geometry) -> int:
+        size = torch.empty((), dtype=geo.dtype).element_size()
+        return n_lines * PagedGroup.pool_pages(PagedGroup.span_of(request), geo) * geo.page_size * request.width * size
+
+    def view(self, line: int, step) -> "CacheLineView":
+        return CacheLineView(group=self, line=line, k=self.k[line], block_table=step.block_tables[self.name])
+
+    def bytes_per_token(self) -> int:
+        return self.n_lines * self.request.width * self.k.element_size()
 
 
 class StateGroup(CacheGroup):
@@ -282,6 +327,7 @@ def _group_type(req) -> type:
 
 
 register_cache_group(KVCacheRequest, KVGroup)
+register_cache_group(LatentCacheRequest, LatentGroup)
 register_cache_group(StateRequest, StateGroup)
 
 
@@ -373,6 +419,8 @@ class Cache:
             name = f"{tag}{sum(1 for g in self.groups if type(g) is kind)}"
             if getattr(req, "window", None) is not None:
                 name += f"w{req.window}"
+            if getattr(req, "chunk", None) is not None:
+                name += f"c{req.chunk}"
             group = kind(name, req, len(entries), geo)
             self.groups.append(group)
             for line, entry in enumerate(entries):
@@ -404,7 +452,7 @@ class Cache:
         sequences at once, so that they lie side by side in the pool as ``grow_together`` wants
         them, and those of the latter piece by piece, between which such a group gives pages back."""
         groups = [g for g in self.kv_groups
-                  if which == "all" or (g.window is None) == (which == "kept")]
+                  if which == "all" or (g.span is None) == (which == "kept")]
         for g in groups:
             need = sum(g.pages_needed(s, n) for s, n in zip(slots, new_lens))
             if need > g.n_free_pages:
@@ -425,7 +473,7 @@ class Cache:
             free = g.n_free_pages
             size: Dict[object, int] = {}
             released: Dict[object, int] = {}
-            w = g.window
+            w = g.span
             for piece in pieces:
                 need = 0
                 for key, n in piece:
@@ -443,7 +491,7 @@ class Cache:
                 free -= need
                 if w is not None:        # what the commit of this piece gives back
                     for key, n in piece:
-                        first_needed = min(max(0, n - w + 1) // g.page_size, size[key])
+                        first_needed = min(g.first_visible(n) // g.page_size, size[key])
                         if first_needed > released[key]:
                             free += first_needed - released[key]
                             released[key] = first_needed

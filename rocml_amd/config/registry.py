@@ -27,6 +27,8 @@ class Architecture:
     read_config: Callable[[Dict], Any]
     to_spec: Callable[[Any], ModelSpec]
     checkpoint_names: Callable[[ModelSpec], Dict[str, str]]
+    # names of tensors a checkpoint may hold although the model does not read them
+    unused_tensors: Callable[[ModelSpec], Any] = lambda spec: ()
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
@@ -85,10 +87,14 @@ def read_config_json(path: str) -> Dict:
 
 
 def architecture_of(raw: Dict) -> Architecture:
+    """The architecture config.json names: the first of ``architectures``, or the string
+    ``architecture``."""
     archs = raw.get("architectures")
-    if not isinstance(archs, (list, tuple)) or not archs:
-        raise ConfigError("config.json lacks the key 'architectures'")
-    return architecture(archs[0])
+    if isinstance(archs, (list, tuple)) and archs:
+        return architecture(archs[0])
+    if isinstance(raw.get("architecture"), str):
+        return architecture(raw["architecture"])
+    raise ConfigError("config.json lacks the key 'architectures' (or 'architecture')")
 
 
 def _register_builtin() -> None:
@@ -98,6 +104,13 @@ def _register_builtin() -> None:
         read_config=qwen3.Qwen3Config.from_dict,
         to_spec=lambda cfg: cfg.to_model_spec(),
         checkpoint_names=qwen3.checkpoint_names))
+    from . import dokulix
+    register_architecture(Architecture(
+        name=dokulix.ARCHITECTURE,
+        read_config=dokulix.DokulixConfig.from_dict,
+        to_spec=lambda cfg: cfg.to_model_spec(),
+        checkpoint_names=dokulix.checkpoint_names,
+        unused_tensors=dokulix.unused_tensors))
 
 
 _register_builtin()

@@ -20,10 +20,12 @@ from typing import Any, Optional, Tuple
 
 @dataclass(frozen=True)
 class NormSpec:
-    """Root-mean-square norm over the last ``size`` values with a gain vector."""
+    """Root-mean-square norm over the last ``size`` values with a gain vector.  ``unit_offset``:
+    the stored weight lies around zero and the gain is one plus it."""
     size: int
     eps: float
     kind: str = "rmsnorm"
+    unit_offset: bool = False
 
 
 @dataclass(frozen=True)
@@ -42,7 +44,14 @@ class AttentionSpec:
 
     ``window`` is ``None`` for full causal attention, else the number of most
     recent positions (the query's own included) a query may see.  ``qk_norm`` is
-    the per-head norm of queries and keys before rotation, or ``None``."""
+    the per-head norm of queries and keys before rotation, or ``None``.
+
+    ``v_head_dim``: the size of a value head when it is not ``head_dim``.  ``bias``: the four
+    projections add a bias vector.  ``chunk``: instead of a window, positions are cut into blocks
+    of so many, counted from position 0, and a query sees the keys of its own block up to itself.
+    ``distance_slopes``: one number per query head; ``slope * (i - j)`` is taken off the score of
+    query ``i`` and key ``j``.  ``sink``: the softmax's denominator has one more term, ``exp(0)``,
+    which has no value."""
     hidden: int
     n_heads: int
     n_kv_heads: int
@@ -52,6 +61,38 @@ class AttentionSpec:
     qk_norm: Optional[NormSpec] = None
     position: Optional[RopeSpec] = None
     kind: str = "attention"
+    v_head_dim: Optional[int] = None
+    bias: bool = False
+    chunk: Optional[int] = None
+    distance_slopes: Optional[Tuple[float, ...]] = None
+    sink: bool = False
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Softmax attention whose keys and values are expanded from one small latent vector per
+    position, which is all the cache holds besides one rotated key part that the heads share.
+
+    Queries: ``c_q = norm(W_dq h)`` (``q_rank`` wide), ``q = W_uq c_q``, per head ``head_dim``
+    values that are not rotated followed by ``rot_dim`` that are.  Keys and values:
+    ``W_dkv h`` gives ``kv_rank`` values, normed into the latent ``c``, and ``rot_dim`` more, the
+    shared rotated key part; per head the unrotated key is ``W_uk c`` and the value ``W_uv c``
+    (``v_head_dim`` wide).  ``gate``: the concatenated heads are multiplied by
+    ``sigmoid(W_g h)`` before the output projection."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    rot_dim: int
+    v_head_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    q_norm: NormSpec
+    kv_norm: NormSpec
+    position: RopeSpec
+    window: Optional[int] = None
+    gate: bool = False
+    kind: str = "latent_attention"
 
 
 @dataclass(frozen=True)
@@ -88,11 +129,12 @@ class BlockSpec:
     """One layer: a mixer and a feed-forward with their norms.
 
     ``arrangement`` names how they are wired; ``pre_norm`` is
-    ``x += mixer(norm(x)); x += ffn(norm(x))``."""
+    ``x += mixer(norm(x)); x += ffn(norm(x))``.  ``ffn`` (and then ``ffn_norm``) may be None:
+    the layer is its mixer alone."""
     mixer: Any
     ffn: Any
     mixer_norm: NormSpec
-    ffn_norm: NormSpec
+    ffn_norm: Optional[NormSpec]
     arrangement: str = "pre_norm"
 
 
@@ -101,9 +143,12 @@ class ScheduleEntry:
     """One execution of a layer.  ``layer`` indexes ``ModelSpec.layers`` (a layer
     may appear in several entries and then runs its weights again with a cache
     line of its own).  ``reads_cache_of`` names an earlier entry of the schedule
-    whose cache line this execution reads instead of writing its own."""
+    whose cache line this execution reads instead of writing its own.  ``offset_row``: row of
+    the model's table of pass offsets (``ModelSpec.pass_offsets`` rows of ``hidden`` values) that
+    is added to the residual stream of every token right before this execution."""
     layer: int
     reads_cache_of: Optional[int] = None
+    offset_row: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -122,6 +167,7 @@ class ModelSpec:
     # table and the norm-then-matrix head that the fields above describe.
     embedding: Any = None
     head: Any = None
+    pass_offsets: int = 0                   # rows of the table that schedule entries add to the stream
 
     def embedding_spec(self) -> Any:
         return self.embedding if self.embedding is not None else \
@@ -139,6 +185,9 @@ class ModelSpec:
             if not 0 <= entry.layer < len(self.layers):
                 raise ConfigError(f"schedule entry {i} names layer {entry.layer}, "
                                   f"the model has {len(self.layers)}")
+            if entry.offset_row is not None and not 0 <= entry.offset_row < self.pass_offsets:
+                raise ConfigError(f"schedule entry {i} adds row {entry.offset_row} of the pass offsets, "
+                                  f"the model has {self.pass_offsets}")
             src = entry.reads_cache_of
             if src is not None:
                 if not 0 <= src < i:

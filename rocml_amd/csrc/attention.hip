@@ -137,7 +137,16 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
                                  int hkv, int d, int page_size, float scale, int window, int algo,
                                  const int* cu_seqlens, int n_seqs, int max_new, const int* q_counts,
                                  int max_len, int n_splits, void* workspace, long long workspace_bytes,
+                                 int dv, int v_in_k, int chunk, const float* slopes, int sink,
                                  hipStream_t stream) {
+    // dv (0: the key head's size), v_in_k, chunk, slopes and sink: see AttnExtra in attention_generic.h.
+    if (dv <= 0) dv = d;
+    ROCML_REQUIRE(chunk >= 0 && (chunk == 0 || window == 0), "attention: a layer has a window or blocks of positions, not both");
+    ROCML_REQUIRE(!v_in_k || dv <= d, "attention: values taken from the key rows need dv <= d (dv=%d d=%d)", dv, d);
+    ROCML_REQUIRE(v_in_k || vcache, "attention: no value cache");
+    ROCML_REQUIRE(dv <= AG_BLOCK * AG_MAX_D_PER_THREAD, "attention: value head size %d exceeds %d", dv,
+                  AG_BLOCK * AG_MAX_D_PER_THREAD);
+    bool plain_features = dv == d && !v_in_k && chunk == 0 && !slopes && !sink;
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0 && page_size > 0 && bt_width > 0,
                   "attention: bad sizes T=%d Hq=%d Hkv=%d D=%d page=%d width=%d", n_tokens, hq, hkv,
                   d, page_size, bt_width);
@@ -158,7 +167,7 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     ROCML_REQUIRE(!q_counts || n_seqs <= 0 || counted == n_tokens,
                   "attention: the sequences' query counts add up to %lld, the step has %d tokens", counted, n_tokens);
     ROCML_REQUIRE(total_q_tiles * hq < (1ll << 31), "attention: too many query tiles");
-    bool mfma_ok = dtype == ROCML_BF16 && page_size == AM_PAGE && mfma_head_dim(d) && max_new >= 1 &&
+    bool mfma_ok = plain_features && dtype == ROCML_BF16 && page_size == AM_PAGE && mfma_head_dim(d) && max_new >= 1 &&
                    (decode ? hq / hkv <= 16 : (cu_seqlens != nullptr && n_seqs > 0 && total_q_tiles > 0));
     if (algo == ATTN_MFMA)
         ROCML_REQUIRE(mfma_ok, "attention: the MFMA kernels need bfloat16, pages of 64 positions, a head size "
@@ -175,14 +184,15 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     }
     dim3 grid(n_tokens, hq);
     size_t lds = (size_t)(d + AG_BLOCK) * sizeof(float);
+    AttnExtra ex{dv, v_in_k, chunk, slopes, sink};
     if (dtype == ROCML_F32)
         attn_generic_kernel<float><<<grid, AG_BLOCK, lds, stream>>>(
             (const float*)q, (float*)out, (const float*)kcache, (const float*)vcache, block_table,
-            bt_width, token_seq, token_pos, hq, hkv, d, page_size, scale, window);
+            bt_width, token_seq, token_pos, hq, hkv, d, page_size, scale, window, ex);
     else if (dtype == ROCML_BF16)
         attn_generic_kernel<bf16_t><<<grid, AG_BLOCK, lds, stream>>>(
             (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,
-            bt_width, token_seq, token_pos, hq, hkv, d, page_size, scale, window);
+            bt_width, token_seq, token_pos, hq, hkv, d, page_size, scale, window, ex);
     else
         return rocml_fail("attention: unknown dtype code %d", dtype);
     ROCML_CHECK_LAUNCH("attention");

@@ -5,7 +5,18 @@
 // scale, running maximum m, l = l * e^(m - m') + sum e^(s - m'), acc likewise, out = acc / l.
 // A query at position p sees keys [lo, p], lo = 0 or p - window + 1.  Keys are taken 256 at a
 // time: every thread scores one key, then the threads split the head's values.
-// Cache layout: keys [page, Hkv, page_size, D], values transposed in a page [page, Hkv, D, page_size].
+// Cache layout: keys [page, Hkv, page_size, D], values transposed in a page [page, Hkv, Dv, page_size].
+//
+// What a layer may add to this, all of it parameters (AttnExtra):
+//  * dv: the size of a value head, when it is not the size of a key head;
+//  * v_in_k: there is no value cache, the value of a key is the first dv numbers of its row (keys
+//    and values expanded from one latent vector, with the expansion folded into the queries and
+//    into the product after the attention: one key/value head [latent, rotated part]);
+//  * chunk: positions are cut into blocks of `chunk`, counted from 0; a query sees its own block
+//    up to itself (lo = pos - pos % chunk) instead of a window;
+//  * slopes[h]: slope * (pos - j) is taken off the score of key j;
+//  * sink: one more term exp(0) in the denominator, with no value: the running maximum starts at 0
+//    and the running sum at 1.
 #pragma once
 #include "common.h"
 
@@ -34,12 +45,25 @@ __device__ __forceinline__ float ag_block_sum(float v, float* scratch) {
     return r;
 }
 
+struct AttnExtra {
+    int dv;                 // value head size
+    int v_in_k;             // values are the leading dv numbers of the key rows
+    int chunk;              // 0: none
+    const float* slopes;    // [Hq] or null
+    int sink;
+};
+
+__device__ __forceinline__ int attn_first_key(int pos, int window, int chunk) {
+    if (chunk > 0) return pos - pos % chunk;
+    return window > 0 ? max(0, pos - window + 1) : 0;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(AG_BLOCK)
 attn_generic_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ kcache,
                     const T* __restrict__ vcache, const int* __restrict__ block_table, int bt_width,
                     const int* __restrict__ token_seq, const int* __restrict__ token_pos, int hq,
-                    int hkv, int d, int page_size, float scale, int window) {
+                    int hkv, int d, int page_size, float scale, int window, AttnExtra ex) {
     extern __shared__ float smem[];
     float* qs = smem;                 // [d]
     float* ps = smem + d;             // [AG_BLOCK]
@@ -48,11 +72,13 @@ attn_generic_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __res
     int pos = token_pos[t];
     const int* pages = block_table + (size_t)token_seq[t] * bt_width;
     int kvh = h / (hq / hkv);
-    int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    int lo = attn_first_key(pos, window, ex.chunk);
+    int dv = ex.dv;
+    float slope = ex.slopes ? ex.slopes[h] : 0.f;
     const T* qrow = q + ((size_t)t * hq + h) * d;
     for (int e = tid; e < d; e += AG_BLOCK) qs[e] = Elem<T>::load(qrow + e);
     __syncthreads();
-    float m = -INFINITY, l = 0.f;
+    float m = ex.sink ? 0.f : -INFINITY, l = ex.sink ? 1.f : 0.f;
     float acc[AG_MAX_D_PER_THREAD] = {};
     for (int c0 = lo; c0 <= pos; c0 += AG_BLOCK) {
         int j = c0 + tid;
@@ -62,7 +88,7 @@ attn_generic_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __res
             const T* krow = kcache + (((size_t)page * hkv + kvh) * page_size + j % page_size) * d;
             float dot = 0.f;
             for (int e = 0; e < d; ++e) dot = fmaf(qs[e], Elem<T>::load(krow + e), dot);
-            s = dot * scale;
+            s = dot * scale - slope * (float)(pos - j);
         }
         float m_new = fmaxf(m, ag_block_max(s, red));
         float corr = expf(m - m_new);            // first chunk: exp(-inf) = 0
@@ -73,23 +99,32 @@ attn_generic_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __res
 #pragma unroll
         for (int r = 0; r < AG_MAX_D_PER_THREAD; ++r) {
             int e = tid + r * AG_BLOCK;
-            if (e >= d) break;
+            if (e >= dv) break;
             float a = acc[r] * corr;
-            for (int jj = 0; jj < n_keys; ++jj) {
-                int key = c0 + jj;
-                int page = pages[key / page_size];
-                const T* vcol = vcache + ((size_t)page * hkv + kvh) * d * page_size + key % page_size;
-                a = fmaf(ps[jj], Elem<T>::load(vcol + (size_t)e * page_size), a);
+            if (ex.v_in_k) {
+                for (int jj = 0; jj < n_keys; ++jj) {
+                    int key = c0 + jj;
+                    int page = pages[key / page_size];
+                    const T* krow = kcache + (((size_t)page * hkv + kvh) * page_size + key % page_size) * d;
+                    a = fmaf(ps[jj], Elem<T>::load(krow + e), a);
+                }
+            } else {
+                for (int jj = 0; jj < n_keys; ++jj) {
+                    int key = c0 + jj;
+                    int page = pages[key / page_size];
+                    const T* vcol = vcache + ((size_t)page * hkv + kvh) * dv * page_size + key % page_size;
+                    a = fmaf(ps[jj], Elem<T>::load(vcol + (size_t)e * page_size), a);
+                }
             }
             acc[r] = a;
         }
         m = m_new;
         __syncthreads();                         // ps is rewritten by the next chunk
     }
-    T* orow = out + ((size_t)t * hq + h) * d;
+    T* orow = out + ((size_t)t * hq + h) * dv;
 #pragma unroll
     for (int r = 0; r < AG_MAX_D_PER_THREAD; ++r) {
         int e = tid + r * AG_BLOCK;
-        if (e < d) Elem<T>::store(orow + e, acc[r] / l);
+        if (e < dv) Elem<T>::store(orow + e, acc[r] / l);
     }
 }

@@ -205,9 +205,16 @@ ROCML_EXPORT int rocml_rmsnorm(float* x, const float* gain, void* out, int out_d
 // (rocml-kernels/kernels/silu_mul.hip:12-20).  Gate and up halves lie side by side in a row.
 // With `interleaved` a row holds (gate_0, up_0, gate_1, up_1, ...), the order the fused product
 // epilogue wants its weight rows in.
+// act: 0 silu, 1 relu (max(g, 0)), 2 gelu with the tanh form 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))).
+__device__ __forceinline__ float gate_activation(float g, int act) {
+    if (act == 1) return fmaxf(g, 0.f);
+    if (act == 2) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.0f + expf(-g));
+}
+
 template <typename TI, typename TO>
 __global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter,
-                              long long total, int interleaved) {
+                              long long total, int interleaved, int act) {
     long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
     if (idx >= total) return;
     long long t = idx / inter;
@@ -215,21 +222,22 @@ __global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, i
     const TI* row = gu + (size_t)t * 2 * inter;
     float g = Elem<TI>::load(row + (interleaved ? 2 * i : i));
     float u = Elem<TI>::load(row + (interleaved ? 2 * i + 1 : inter + i));
-    Elem<TO>::store(out + idx, g / (1.0f + expf(-g)) * u);
+    Elem<TO>::store(out + idx, gate_activation(g, act) * u);
 }
 
 ROCML_EXPORT int rocml_swiglu(const void* gu, int in_dtype, void* out, int out_dtype, int n_tokens,
-                              int inter, int interleaved, hipStream_t stream) {
+                              int inter, int interleaved, int act, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
+    ROCML_REQUIRE(act >= 0 && act <= 2, "swiglu: unknown activation %d (0 silu, 1 relu, 2 gelu_tanh)", act);
     long long total = (long long)n_tokens * inter;
     if (total == 0) return 0;
     int grid = ceil_div(total, EW_BLOCK);
     if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32)
-        swiglu_kernel<float, float><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (float*)out, inter, total, interleaved);
+        swiglu_kernel<float, float><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (float*)out, inter, total, interleaved, act);
     else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16)
-        swiglu_kernel<float, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (bf16_t*)out, inter, total, interleaved);
+        swiglu_kernel<float, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (bf16_t*)out, inter, total, interleaved, act);
     else if (in_dtype == ROCML_BF16 && out_dtype == ROCML_BF16)
-        swiglu_kernel<bf16_t, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, interleaved);
+        swiglu_kernel<bf16_t, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, interleaved, act);
     else
         return rocml_fail("swiglu: unsupported dtype pair in=%d out=%d", in_dtype, out_dtype);
     ROCML_CHECK_LAUNCH("swiglu");
@@ -285,7 +293,9 @@ __global__ void qk_norm_rope_append_kernel(
     TO* __restrict__ q_out, TO* __restrict__ kcache, TO* __restrict__ vcache,
     const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
     const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride,
-    int rows_per_token, int pairing, int first_row) {
+    int rows_per_token, int pairing, int first_row, const float* __restrict__ bias, int dv) {
+    // bias (may be null): one number per column of the packed row, added to the projection's sums.
+    // dv: the size of a value head; the value rows start behind the Hq + Hkv rows of d numbers.
     extern __shared__ float stage[];   // [QK_WAVES][d]
     int wave = threadIdx.x / WAVE;
     int lane = threadIdx.x & (WAVE - 1);
@@ -295,14 +305,17 @@ __global__ void qk_norm_rope_append_kernel(
     int r = first_row + (active ? (int)(row - (long long)t * rows_per_token) : 0);     // first_row = hq: no q rows
     int kind = r < hq ? 0 : (r < hq + hkv ? 1 : 2);   // q, k, v
     if (!write_kv && kind != 0) active = false;
-    const TI* src = qkv + (size_t)t * ld + (size_t)r * d;
+    int width = kind == 2 ? dv : d;
+    size_t col0 = kind == 2 ? (size_t)(hq + hkv) * d + (size_t)(r - hq - hkv) * dv : (size_t)r * d;
+    const TI* src = qkv + (size_t)t * ld + col0;
     float v[QK_PER_LANE];
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < QK_PER_LANE; ++j) {
         int e = lane + j * WAVE;
-        bool ok = active && e < d;
+        bool ok = active && e < width;
         float val = Elem<TI>::load(ok ? src + e : qkv);
+        if (bias && ok) val += bias[col0 + e];
         // split-K partial sums of the projection, added in split order
         // (four loads in flight at a time)
         for (int sp = 1; sp < n_splits; sp += 4) {
@@ -383,12 +396,12 @@ __global__ void qk_norm_rope_append_kernel(
         int page = block_table[(size_t)token_seq[t] * bt_width + pos / page_size];
         if (page < 0) return;
         if (kind == 2) {
-            // values are stored transposed inside a page: [page, Hkv, D, page_size]
-            TO* vdst = vcache + ((size_t)page * hkv + head) * d * page_size + pos % page_size;
+            // values are stored transposed inside a page: [page, Hkv, Dv, page_size]
+            TO* vdst = vcache + ((size_t)page * hkv + head) * dv * page_size + pos % page_size;
 #pragma unroll
             for (int j = 0; j < QK_PER_LANE; ++j) {
                 int e = lane + j * WAVE;
-                if (e < d) Elem<TO>::store(vdst + (size_t)e * page_size, v[j]);
+                if (e < dv) Elem<TO>::store(vdst + (size_t)e * page_size, v[j]);
             }
             return;
         }
@@ -483,7 +496,8 @@ template <typename TI, typename TO>
 __global__ void __launch_bounds__(EW_BLOCK)
 v_append_tile_kernel(const TI* __restrict__ qkv, int ld, int n_tokens, int v_col0, int hkv, int d,
                      TO* __restrict__ vcache, const int* __restrict__ block_table, int bt_width,
-                     const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size) {
+                     const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size,
+                     const float* __restrict__ bias) {
     __shared__ float vt_stage[VT_TOKENS][VT_VALUES + 1];
     int t0 = blockIdx.x * VT_TOKENS, head = blockIdx.y, e0 = blockIdx.z * VT_VALUES;
     int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
@@ -493,6 +507,7 @@ v_append_tile_kernel(const TI* __restrict__ qkv, int ld, int n_tokens, int v_col
     for (int i = 0; i < VT_TOKENS * VT_VALUES / EW_BLOCK; ++i) {
         int j = min(t0 + (tid >> 5) + (EW_BLOCK / VT_VALUES) * i, n_tokens - 1), e = min(e0 + (tid & 31), d - 1);
         tmp[i] = Elem<TI>::load(qkv + (size_t)j * ld + v_col0 + (size_t)head * d + e);
+        if (bias) tmp[i] += bias[v_col0 + (size_t)head * d + e];
     }
 #pragma unroll
     for (int i = 0; i < VT_TOKENS * VT_VALUES / EW_BLOCK; ++i) vt_stage[(tid >> 5) + (EW_BLOCK / VT_VALUES) * i][tid & 31] = tmp[i];
@@ -515,13 +530,17 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, int pairing, void* q_out,
     void* kcache, void* vcache, int out_dtype, const int* block_table, int bt_width,
     const int* token_seq, const int* token_pos, int page_size, int write_kv, int n_splits,
-    long long split_stride, hipStream_t stream) {
+    long long split_stride, const float* bias, int dv, hipStream_t stream) {
+    // bias (may be null): [ld] numbers added to the projection's sums; dv (0: d): value head size.
+    if (dv <= 0) dv = d;
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0, "qk_norm_rope_append: bad sizes");
+    ROCML_REQUIRE(dv <= QK_MAX_PER_LANE * WAVE, "qk_norm_rope_append: value head size %d exceeds %d", dv,
+                  QK_MAX_PER_LANE * WAVE);
     ROCML_REQUIRE(n_splits >= 1 && (n_splits == 1 || (split_stride > 0 && in_dtype == ROCML_F32)),
                   "qk_norm_rope_append: partial sums must be 32-bit with a positive stride");
     ROCML_REQUIRE(d <= QK_MAX_PER_LANE * WAVE, "qk_norm_rope_append: head_dim %d exceeds %d", d,
                   QK_MAX_PER_LANE * WAVE);
-    ROCML_REQUIRE(ld >= (hq + 2 * hkv) * d || (!write_kv && ld >= hq * d),
+    ROCML_REQUIRE(ld >= (hq + hkv) * d + hkv * dv || (!write_kv && ld >= hq * d),
                   "qk_norm_rope_append: row stride %d too small", ld);
     ROCML_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope_append: rot_dim %d must be even and <= %d", rot, d);
     ROCML_REQUIRE(pairing == 0 || pairing == 1, "qk_norm_rope_append: pairing %d (0: halves, 1: neighbours)", pairing);
@@ -536,12 +555,13 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     int first_row = q_out ? 0 : hq;
     int rows_per_token = hq - first_row + (write_kv ? (v_tiled ? hkv : 2 * hkv) : 0);
     long long rows = (long long)n_tokens * rows_per_token;
-    int per_lane = d <= 64 ? 1 : d <= 128 ? 2 : d <= 256 ? 4 : 8;     // head values per lane
+    int widest = d > dv ? d : dv;
+    int per_lane = widest <= 64 ? 1 : widest <= 128 ? 2 : widest <= 256 ? 4 : 8;     // head values per lane
     // both values of a rotation pair in one lane: whole head rotated, d = per_lane * 64
     // (and the pairs are (e, e + d/2): neighbours as pairs go through LDS)
-    bool local_pair = per_lane >= 2 && (rot == 0 || (rot == d && pairing == 0)) && d == per_lane * WAVE;
+    bool local_pair = per_lane >= 2 && (rot == 0 || (rot == d && pairing == 0)) && d == per_lane * WAVE && dv == d;
     // many rows, none of them values: several rows per wave
-    bool many_rows = local_pair && per_lane <= 4 && n_splits == 1 && n_tokens >= VT_TOKENS && (v_tiled || !write_kv);
+    bool many_rows = !bias && local_pair && per_lane <= 4 && n_splits == 1 && n_tokens >= VT_TOKENS && (v_tiled || !write_kv);
     constexpr int MANY = 4;
     int grid = many_rows ? ceil_div(rows, QK_WAVES * MANY) : ceil_div(rows, QK_WAVES);
     size_t lds = local_pair ? 0 : (size_t)QK_WAVES * d * sizeof(float);
@@ -549,7 +569,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     qk_norm_rope_append_kernel<TI, TO, N, LP><<<grid, EW_BLOCK, lds, stream>>>(                 \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
-        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row)
+        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row, bias, dv)
 #define LAUNCH_ROWS(TI, TO, N)                                                                  \
     qk_norm_rope_rows_kernel<TI, TO, N, MANY><<<grid, EW_BLOCK, 0, stream>>>(                   \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, rot ? cos_t : nullptr,   \
@@ -563,10 +583,10 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
         else if (per_lane == 4) { if (local_pair) LAUNCH_N(TI, TO, 4, true); else LAUNCH_N(TI, TO, 4, false); } \
         else { if (local_pair) LAUNCH_N(TI, TO, 8, true); else LAUNCH_N(TI, TO, 8, false); }    \
         if (v_tiled) {                                                                          \
-            dim3 vgrid(ceil_div(n_tokens, VT_TOKENS), hkv, ceil_div(d, VT_VALUES));             \
+            dim3 vgrid(ceil_div(n_tokens, VT_TOKENS), hkv, ceil_div(dv, VT_VALUES));            \
             v_append_tile_kernel<TI, TO><<<vgrid, EW_BLOCK, 0, stream>>>(                       \
-                (const TI*)qkv, ld, n_tokens, (hq + hkv) * d, hkv, d, (TO*)vcache, block_table, \
-                bt_width, token_seq, token_pos, page_size);                                     \
+                (const TI*)qkv, ld, n_tokens, (hq + hkv) * d, hkv, dv, (TO*)vcache, block_table,\
+                bt_width, token_seq, token_pos, page_size, bias);                               \
         }                                                                                       \
     }
     if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32) LAUNCH(float, float)
@@ -597,5 +617,179 @@ ROCML_EXPORT int rocml_add_into(float* x, const void* y, int y_dtype, long long 
     else if (y_dtype == ROCML_BF16) add_into_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>(x, (const bf16_t*)y, total);
     else return rocml_fail("add_into: unknown dtype code %d", y_dtype);
     ROCML_CHECK_LAUNCH("add_into");
+    return 0;
+}
+
+// ---- a vector added to every row -------------------------------------------------
+// x[t, :] += b: a projection's bias on the way into the residual stream, or a table row that a
+// schedule entry adds to the stream before it runs.
+__global__ void add_row_vector_kernel(float* __restrict__ x, const float* __restrict__ b, int n, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx < total) x[idx] += b[idx % n];
+}
+
+ROCML_EXPORT int rocml_add_row_vector(float* x, const float* b, int n_rows, int n, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && n > 0, "add_row_vector: bad sizes rows=%d n=%d", n_rows, n);
+    long long total = (long long)n_rows * n;
+    if (total == 0) return 0;
+    add_row_vector_kernel<<<ceil_div(total, EW_BLOCK), EW_BLOCK, 0, stream>>>(x, b, n, total);
+    ROCML_CHECK_LAUNCH("add_row_vector");
+    return 0;
+}
+
+// ---- latent attention: what follows the first projection ---------------------------
+// A token's row of the projection holds, side by side, q_rank numbers (the query latent),
+// kv_rank numbers (the key/value latent), rot_part numbers (the key part that is rotated and
+// shared by the heads) and whatever else the caller projected with the same product (a gate).
+// One block per token: both latents are divided by their root mean square (32-bit, eps inside the
+// root) and multiplied by their gains; the query latent goes to cq_out, the key/value latent and
+// the rotated key part go into the token's row of the paged cache [page, page_size, kv_rank +
+// rot_part].  Rotation: pairs (i, i + dims/2) of the first `dims` numbers of the part by the
+// angle in column i of the tables [T, dims/2]; the rest of the part passes unchanged.
+__device__ __forceinline__ float block_sum_256(float v, float* scratch) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & (WAVE - 1)) == 0) scratch[threadIdx.x / WAVE] = v;
+    __syncthreads();
+    float r = 0.f;
+#pragma unroll
+    for (int w = 0; w < EW_BLOCK / WAVE; ++w) r += scratch[w];
+    return r;
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(EW_BLOCK)
+latent_prepare_kernel(const float* __restrict__ proj, int ld, int q_rank, int kv_rank, int rot_part, int dims,
+                      const float* __restrict__ q_gain, const float* __restrict__ kv_gain, float eps,
+                      const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                      TO* __restrict__ cq_out, TO* __restrict__ cache, const int* __restrict__ block_table,
+                      int bt_width, const int* __restrict__ token_seq, const int* __restrict__ token_pos,
+                      int page_size, int write_cache) {
+    __shared__ float red[EW_BLOCK / WAVE];
+    int t = blockIdx.x, tid = threadIdx.x;
+    const float* row = proj + (size_t)t * ld;
+    float sq = 0.f, sk = 0.f;
+    for (int e = tid; e < q_rank; e += EW_BLOCK) sq = fmaf(row[e], row[e], sq);
+    for (int e = tid; e < kv_rank; e += EW_BLOCK) sk = fmaf(row[q_rank + e], row[q_rank + e], sk);
+    float inv_q = 1.0f / sqrtf(block_sum_256(sq, red) / (float)q_rank + eps);
+    float inv_k = 1.0f / sqrtf(block_sum_256(sk, red) / (float)kv_rank + eps);
+    for (int e = tid; e < q_rank; e += EW_BLOCK)
+        Elem<TO>::store(cq_out + (size_t)t * q_rank + e, row[e] * inv_q * q_gain[e]);
+    if (!write_cache) return;
+    int pos = token_pos[t];
+    int page = block_table[(size_t)token_seq[t] * bt_width + pos / page_size];
+    if (page < 0) return;
+    TO* dst = cache + ((size_t)page * page_size + pos % page_size) * (kv_rank + rot_part);
+    for (int e = tid; e < kv_rank; e += EW_BLOCK)
+        Elem<TO>::store(dst + e, row[q_rank + e] * inv_k * kv_gain[e]);
+    const float* kr = row + q_rank + kv_rank;
+    int half = dims / 2;
+    for (int e = tid; e < rot_part; e += EW_BLOCK) {
+        float v = kr[e];
+        if (e < half) {
+            float c = cos_t[(size_t)t * half + e], s = sin_t[(size_t)t * half + e];
+            v = kr[e] * c - kr[e + half] * s;
+        } else if (e < dims) {
+            float c = cos_t[(size_t)t * half + e - half], s = sin_t[(size_t)t * half + e - half];
+            v = kr[e] * c + kr[e - half] * s;
+        }
+        Elem<TO>::store(dst + kv_rank + e, v);
+    }
+}
+
+ROCML_EXPORT int rocml_latent_prepare(const float* proj, int ld, int n_tokens, int q_rank, int kv_rank, int rot_part,
+                                      int dims, const float* q_gain, const float* kv_gain, float eps,
+                                      const float* cos_t, const float* sin_t, void* cq_out, void* cache,
+                                      int out_dtype, const int* block_table, int bt_width, const int* token_seq,
+                                      const int* token_pos, int page_size, int write_cache, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && q_rank > 0 && kv_rank > 0 && rot_part >= 0 && dims >= 0 && dims % 2 == 0 && dims <= rot_part,
+                  "latent_prepare: bad sizes T=%d q_rank=%d kv_rank=%d rotated part=%d of which %d turn", n_tokens,
+                  q_rank, kv_rank, rot_part, dims);
+    ROCML_REQUIRE(ld >= q_rank + kv_rank + rot_part, "latent_prepare: rows of %d numbers, %d are needed", ld,
+                  q_rank + kv_rank + rot_part);
+    ROCML_REQUIRE(q_gain && kv_gain && cq_out && (dims == 0 || (cos_t && sin_t)), "latent_prepare: gains, tables or output missing");
+    ROCML_REQUIRE(!write_cache || (cache && block_table && bt_width > 0 && page_size > 0 && token_seq && token_pos),
+                  "latent_prepare: cache arguments missing");
+    if (n_tokens == 0) return 0;
+#define LAUNCH(TO)                                                                                              \
+    latent_prepare_kernel<TO><<<n_tokens, EW_BLOCK, 0, stream>>>(proj, ld, q_rank, kv_rank, rot_part, dims,    \
+        q_gain, kv_gain, eps, cos_t, sin_t, (TO*)cq_out, (TO*)cache, block_table, bt_width, token_seq,         \
+        token_pos, page_size, write_cache)
+    if (out_dtype == ROCML_F32) LAUNCH(float);
+    else if (out_dtype == ROCML_BF16) LAUNCH(bf16_t);
+    else return rocml_fail("latent_prepare: unknown dtype code %d", out_dtype);
+#undef LAUNCH
+    ROCML_CHECK_LAUNCH("latent_prepare");
+    return 0;
+}
+
+// The rotated part of every query head: q [T, ldq] holds, per head, head_stride numbers of which
+// those from `offset` on, rot_part of them, are the part; its rotation (as above) goes to
+// out [T, ldo] at out_offset of each head's out_stride numbers.
+template <typename TO>
+__global__ void rope_heads_kernel(const float* __restrict__ q, int ldq, int head_stride, int offset, int rot_part,
+                                  int dims, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                  TO* __restrict__ out, int ldo, int out_stride, int out_offset, int n_heads,
+                                  long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    int e = (int)(idx % rot_part);
+    long long th = idx / rot_part;
+    int h = (int)(th % n_heads);
+    long long t = th / n_heads;
+    const float* src = q + (size_t)t * ldq + (size_t)h * head_stride + offset;
+    int half = dims / 2;
+    float v = src[e];
+    if (e < half) {
+        v = src[e] * cos_t[t * half + e] - src[e + half] * sin_t[t * half + e];
+    } else if (e < dims) {
+        v = src[e] * cos_t[t * half + e - half] + src[e - half] * sin_t[t * half + e - half];
+    }
+    Elem<TO>::store(out + (size_t)t * ldo + (size_t)h * out_stride + out_offset + e, v);
+}
+
+ROCML_EXPORT int rocml_rope_heads(const float* q, int ldq, int head_stride, int offset, int rot_part, int dims,
+                                  const float* cos_t, const float* sin_t, void* out, int out_dtype, int ldo,
+                                  int out_stride, int out_offset, int n_tokens, int n_heads, hipStream_t stream) {
+    ROCML_REQUIRE(n_tokens >= 0 && n_heads > 0 && rot_part >= 0 && dims >= 0 && dims % 2 == 0 && dims <= rot_part,
+                  "rope_heads: bad sizes T=%d H=%d part=%d dims=%d", n_tokens, n_heads, rot_part, dims);
+    ROCML_REQUIRE(offset >= 0 && offset + rot_part <= head_stride && ldq >= n_heads * head_stride &&
+                      out_offset >= 0 && out_offset + rot_part <= out_stride && ldo >= n_heads * out_stride,
+                  "rope_heads: the part does not lie inside the heads");
+    ROCML_REQUIRE(dims == 0 || (cos_t && sin_t), "rope_heads: rotation tables missing");
+    long long total = (long long)n_tokens * n_heads * rot_part;
+    if (total == 0) return 0;
+    int grid = ceil_div(total, EW_BLOCK);
+    if (out_dtype == ROCML_F32)
+        rope_heads_kernel<float><<<grid, EW_BLOCK, 0, stream>>>(q, ldq, head_stride, offset, rot_part, dims, cos_t, sin_t,
+                                                                (float*)out, ldo, out_stride, out_offset, n_heads, total);
+    else if (out_dtype == ROCML_BF16)
+        rope_heads_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>(q, ldq, head_stride, offset, rot_part, dims, cos_t, sin_t,
+                                                                 (bf16_t*)out, ldo, out_stride, out_offset, n_heads, total);
+    else return rocml_fail("rope_heads: unknown dtype code %d", out_dtype);
+    ROCML_CHECK_LAUNCH("rope_heads");
+    return 0;
+}
+
+// y[t, i] = y[t, i] * sigmoid(g[t, i]) with g 32-bit in rows of ldg numbers: an output gate.
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ y, const float* __restrict__ g, int ldg, int n, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    long long t = idx / n;
+    int i = (int)(idx - t * n);
+    float gate = 1.0f / (1.0f + expf(-g[(size_t)t * ldg + i]));
+    Elem<T>::store(y + idx, Elem<T>::load(y + idx) * gate);
+}
+
+ROCML_EXPORT int rocml_sigmoid_gate(void* y, int dtype, const float* g, int ldg, int n_rows, int n, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && n > 0 && ldg >= n, "sigmoid_gate: bad sizes rows=%d n=%d ld=%d", n_rows, n, ldg);
+    long long total = (long long)n_rows * n;
+    if (total == 0) return 0;
+    int grid = ceil_div(total, EW_BLOCK);
+    if (dtype == ROCML_F32) sigmoid_gate_kernel<float><<<grid, EW_BLOCK, 0, stream>>>((float*)y, g, ldg, n, total);
+    else if (dtype == ROCML_BF16) sigmoid_gate_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>((bf16_t*)y, g, ldg, n, total);
+    else return rocml_fail("sigmoid_gate: unknown dtype code %d", dtype);
+    ROCML_CHECK_LAUNCH("sigmoid_gate");
     return 0;
 }

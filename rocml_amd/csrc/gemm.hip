@@ -101,7 +101,7 @@ static double tile_cost(const TileKind& kind, int pieces, int m, int n, int k, i
     double pulled = (double)(kind.bn + (m < kind.bm ? m : kind.bm)) * k_per_piece * 2.0 * (double)ceil_div(blocks, (long long)cus);
     if (t < pulled / 36.0e3) t = pulled / 36.0e3;
     t += 3.0;
-    double moved = epi == EPI_SWIGLU ? (double)m * n
+    double moved = epi_gated(epi) ? (double)m * n
                    : pieces > 1      ? (double)m * n * 4.0 * pieces
                                      : (double)m * n * 4.0 * (epi == EPI_ACC ? 2.0 : 1.0);
     t += moved / 2.0e6;
@@ -127,7 +127,7 @@ static int launch_mfma_tile(const void* x, int ldx, const void* w, int ldw, void
         double best = 1e30;
         for (const auto& kind : TILE_KINDS) {
             for (int pieces = 1; pieces <= 8 && pieces <= plan.max_splits; ++pieces) {
-                if (pieces > 1 && (EPI == EPI_SWIGLU || k / pieces < 256 || !workspace ||
+                if (pieces > 1 && (epi_gated(EPI) || k / pieces < 256 || !workspace ||
                                    (long long)pieces * m * n * (long long)sizeof(float) > workspace_bytes))
                     break;
                 double t = tile_cost(kind, pieces, m, n, k, EPI, cus);
@@ -271,7 +271,7 @@ template <int MT, int EPI>
 static int launch_skinny(const void* x, int ldx, const void* w, int ldw, void* out, int ldo, int m, int n,
                          int k, void* workspace, long long workspace_bytes, SplitPlan plan, hipStream_t stream) {
     const int cus = cu_count();
-    if constexpr (EPI == EPI_SWIGLU) {
+    if constexpr (epi_gated(EPI)) {
         // The gated epilogue needs whole sums: the kernel that requests two steps ahead, whatever
         // the number of rows, with the number of waves that makes its blocks one round.  (At 49 to
         // 64 rows the kernels of 13 to 15 waves need more registers than 832 to 960 threads
@@ -386,7 +386,7 @@ static int launch_kpar(const void* x, int ldx, const void* w, int ldw, void* out
     int by_k = k / 1024;
     if (splits > by_k) splits = by_k;
     if (splits > plan.max_splits) splits = plan.max_splits;
-    if (splits < 1 || EPI == EPI_SWIGLU) splits = 1;
+    if (splits < 1 || epi_gated(EPI)) splits = 1;
     long long per_split = (long long)m * n * sizeof(float);
     if (splits > 1 && (long long)splits * per_split > workspace_bytes)
         splits = workspace ? (int)(workspace_bytes / per_split) : 1;
@@ -423,12 +423,12 @@ static int launch_skinny_m(const void* x, int ldx, const void* w, int ldw, void*
 // Gated activation over a 32-bit [M, N] product with (gate, up) column pairs: the unfused path of
 // the epilogue above, for the kernels that cannot fuse it.
 template <typename TO>
-__global__ void swiglu_pairs_kernel(const float* __restrict__ gu, TO* __restrict__ out, int ldo, int m, int half) {
+__global__ void swiglu_pairs_kernel(const float* __restrict__ gu, TO* __restrict__ out, int ldo, int m, int half, int relu) {
     long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (long long)m * half) return;
     int r = (int)(idx / half), j = (int)(idx - (long long)r * half);
     const float* row = gu + (size_t)r * 2 * half;
-    Elem<TO>::store(out + (size_t)r * ldo + j, silu_mul(row[2 * j], row[2 * j + 1]));
+    Elem<TO>::store(out + (size_t)r * ldo + j, relu ? fmaxf(row[2 * j], 0.f) * row[2 * j + 1] : silu_mul(row[2 * j], row[2 * j + 1]));
 }
 
 // out (+)= sum of split-K partial sums [splits][M][N] in split order: the step that a deferred
@@ -521,8 +521,8 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
                             int max_splits, hipStream_t stream) {
     if (deferred_splits) *deferred_splits = 0;
     ROCML_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm: bad sizes M=%d N=%d K=%d", m, n, k);
-    bool gated = epilogue == 1;
-    ROCML_REQUIRE(epilogue == 0 || epilogue == 1, "gemm: unknown epilogue %d", epilogue);
+    bool gated = epilogue == 1 || epilogue == 2;        // 1: silu(gate) * up, 2: max(gate, 0) * up
+    ROCML_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm: unknown epilogue %d", epilogue);
     ROCML_REQUIRE(!gated || (n % 2 == 0 && !accumulate), "gemm: the gated epilogue needs an even N and no accumulation");
     int out_cols = gated ? n / 2 : n;
     ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= out_cols, "gemm: row strides (%d, %d, %d) below (K, K, N)",
@@ -542,7 +542,7 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     if (algo == ALGO_MFMA_KPAR)
         ROCML_REQUIRE(m <= 16, "gemm: the 16-rows kernel takes at most 16 rows, got %d", m);
     ROCML_REQUIRE(out_dtype == ROCML_F32 || out_dtype == ROCML_BF16, "gemm: unknown output type %d", out_dtype);
-    int epi = gated ? EPI_SWIGLU : accumulate ? EPI_ACC : (out_dtype == ROCML_BF16 ? EPI_BF16 : EPI_F32);
+    int epi = gated ? (epilogue == 2 ? EPI_RELUGLU : EPI_SWIGLU) : accumulate ? EPI_ACC : (out_dtype == ROCML_BF16 ? EPI_BF16 : EPI_F32);
     bool use_mfma = mfma_ok && algo != ALGO_PLAIN;
     if (row_ssq)
         ROCML_REQUIRE(gated && m <= 16 && use_mfma && row_parts > 0 && row_eps > 0.f &&
@@ -564,7 +564,8 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
 #define BY_EPI(fn, ...)                                              \
         (epi == EPI_F32 ? fn<EPI_F32>(__VA_ARGS__)                   \
          : epi == EPI_BF16 ? fn<EPI_BF16>(__VA_ARGS__)               \
-         : epi == EPI_ACC ? fn<EPI_ACC>(__VA_ARGS__) : fn<EPI_SWIGLU>(__VA_ARGS__))
+         : epi == EPI_ACC ? fn<EPI_ACC>(__VA_ARGS__)                 \
+         : epi == EPI_RELUGLU ? fn<EPI_RELUGLU>(__VA_ARGS__) : fn<EPI_SWIGLU>(__VA_ARGS__))
         // One or two rows (but not the gated product, which has its own choice of blocks): the
         // kernel whose waves split K, unless the output is narrow (fewer than
         // one and a half blocks of 16 weight rows a CU: 4096 or 5120 wide on 256 CUs, the products
@@ -608,10 +609,33 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     if (gated) {
         long long total = (long long)m * (n / 2);
         if (out_dtype == ROCML_F32)
-            swiglu_pairs_kernel<float><<<ceil_div(total, 256), 256, 0, stream>>>((const float*)dst, (float*)out, ldo, m, n / 2);
+            swiglu_pairs_kernel<float><<<ceil_div(total, 256), 256, 0, stream>>>((const float*)dst, (float*)out, ldo, m, n / 2, epilogue == 2);
         else
-            swiglu_pairs_kernel<bf16_t><<<ceil_div(total, 256), 256, 0, stream>>>((const float*)dst, (bf16_t*)out, ldo, m, n / 2);
+            swiglu_pairs_kernel<bf16_t><<<ceil_div(total, 256), 256, 0, stream>>>((const float*)dst, (bf16_t*)out, ldo, m, n / 2, epilogue == 2);
     }
     ROCML_CHECK_LAUNCH("gemm");
+    return 0;
+}
+
+// A batch of small products that share their shapes: out_b[M, N] = x_b[M, K] * w_b[N, K]^T for
+// b = 0 .. batch-1, operands and results `batch_*` elements apart (the heads of a layer: x and out
+// are column ranges of wider matrices, w is [batch, N, K]).  32-bit accumulation by fused
+// multiply-add in K order for every type; x may be 32-bit while w is bfloat16.
+ROCML_EXPORT int rocml_gemm_batched(const void* x, int x_dtype, int ldx, long long batch_x, const void* w, int w_dtype,
+                                    int ldw, long long batch_w, void* out, int out_dtype, int ldo, long long batch_o,
+                                    int batch, int m, int n, int k, hipStream_t stream) {
+    ROCML_REQUIRE(batch > 0 && batch < 65536 && m >= 0 && n > 0 && k > 0, "gemm_batched: bad sizes batch=%d M=%d N=%d K=%d", batch, m, n, k);
+    ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= n && batch_x >= 0 && batch_w >= 0 && batch_o >= 0,
+                  "gemm_batched: row strides (%d, %d, %d) below (K, K, N) or a negative batch stride", ldx, ldw, ldo);
+    ROCML_REQUIRE(ceil_div(m, GT_BM) < 65536, "gemm_batched: too many rows %d", m);
+    if (m == 0) return 0;
+#define GB(TX, TW, TO) launch_gemm_tile_batched<TX, TW, TO>(x, ldx, batch_x, w, ldw, batch_w, out, ldo, batch_o, batch, m, n, k, stream)
+    if (x_dtype == ROCML_F32 && w_dtype == ROCML_F32 && out_dtype == ROCML_F32) GB(float, float, float);
+    else if (x_dtype == ROCML_F32 && w_dtype == ROCML_BF16 && out_dtype == ROCML_BF16) GB(float, bf16_t, bf16_t);
+    else if (x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16 && out_dtype == ROCML_BF16) GB(bf16_t, bf16_t, bf16_t);
+    else if (x_dtype == ROCML_BF16 && w_dtype == ROCML_BF16 && out_dtype == ROCML_F32) GB(bf16_t, bf16_t, float);
+    else return rocml_fail("gemm_batched: unsupported type triple x=%d w=%d out=%d", x_dtype, w_dtype, out_dtype);
+#undef GB
+    ROCML_CHECK_LAUNCH("gemm_batched");
     return 0;
 }

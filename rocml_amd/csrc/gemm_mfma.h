@@ -43,9 +43,18 @@ __device__ __forceinline__ bf16x8_t as_frag4(u32x4_t v) { return __builtin_bit_c
 // EPI_SWIGLU: weight rows come in pairs (gate_j, up_j); the output is bfloat16 [M, N/2] with
 // out[m][j] = silu(gate) * up (rocml-kernels/kernels/silu_mul.hip:12-20), formed from the 32-bit
 // accumulators so that gate and up are never rounded or written.
-enum GemmEpilogue : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_ACC = 2, EPI_SWIGLU = 3 };
+// EPI_RELUGLU: the same with max(gate, 0) * up.
+enum GemmEpilogue : int { EPI_F32 = 0, EPI_BF16 = 1, EPI_ACC = 2, EPI_SWIGLU = 3, EPI_RELUGLU = 4 };
+
+constexpr bool epi_gated(int epi) { return epi == EPI_SWIGLU || epi == EPI_RELUGLU; }
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
+template <int EPI>
+__device__ __forceinline__ float gated_mul(float g, float u) {
+    if (EPI == EPI_RELUGLU) return fmaxf(g, 0.f) * u;
+    return silu_mul(g, u);
+}
 
 // The scale of a norm whose product-side half was done by the producer of the residual stream
 // (gemm_residual_prescale_kernel): the operand is bfloat16(x * gain), and the sums of this product
@@ -212,7 +221,7 @@ __device__ __forceinline__ void tile_epilogue(f32x16_t (&acc)[T::TM][T::TN], voi
 #pragma unroll
         for (int j = 0; j < T::TN; ++j) {
             int gn = n0 + (wn * T::TN + j) * 32 + (lane & 31);
-            if (EPI == EPI_SWIGLU) {
+            if (epi_gated(EPI)) {
                 // Neighbouring lanes hold neighbouring columns: the even one the gate, the odd one
                 // the up value of one output column.  Of two neighbouring rows the even lane
                 // finishes the first and the odd lane the second: one exchange per pair of rows,
@@ -225,7 +234,7 @@ __device__ __forceinline__ void tile_epilogue(f32x16_t (&acc)[T::TM][T::TN], voi
                     float gate = odd ? got : first, up = odd ? second : got;
                     int gm = m0 + (wm * T::TM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3) + (odd ? 1 : 0);
                     if (gm < m && (gn | 1) < n)
-                        ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(silu_mul(gate, up));
+                        ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] = f32_to_bf16(gated_mul<EPI>(gate, up));
                 }
                 continue;
             }
@@ -388,14 +397,14 @@ __device__ __forceinline__ void skinny_epilogue(const f32x4_t (&acc)[MT], void* 
     for (int mt = 0; mt < MT; ++mt) {
         int gm = mt * 16 + (lane & 15);
         if (gm >= m) continue;
-        if (EPI == EPI_SWIGLU && !PARTIAL) {
+        if (epi_gated(EPI) && !PARTIAL) {
             // a lane holds weight rows 4g .. 4g+3 = two (gate, up) pairs
 #pragma unroll
             for (int e = 0; e < 4; e += 2) {
                 int gn = n0 + (lane >> 4) * 4 + e;
                 if (gn + 1 < n)
                     ((bf16_t*)out)[(size_t)gm * ldo + (gn >> 1)] =
-                        f32_to_bf16(silu_mul(acc[mt][e] * row_scale, acc[mt][e + 1] * row_scale));
+                        f32_to_bf16(gated_mul<EPI>(acc[mt][e] * row_scale, acc[mt][e + 1] * row_scale));
             }
             continue;
         }
@@ -610,7 +619,7 @@ gemm_skinny_ahead_kernel(const bf16_t* x, int ldx, const bf16_t* w, int ldw, voi
     // The rows' scales, if the operand lacks them (the gated epilogue of at most 16 rows applies
     // them): the block's first waves form them, four rows each, while the first weights are on
     // their way and leave them in LDS for the epilogue.
-    constexpr bool SCALES = MT == 1 && EPI == EPI_SWIGLU && !PARTIAL;
+    constexpr bool SCALES = MT == 1 && epi_gated(EPI) && !PARTIAL;
     __shared__ float ga_scale[16];
     __shared__ __attribute__((aligned(16))) float ga_red[SCALES ? 16 * RS_RED_STRIDE : 4];
     constexpr int SCALE_WAVES = WAVES >= 4 ? 4 : 2, SCALE_ROWS = 16 / SCALE_WAVES;
@@ -695,7 +704,7 @@ gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     if (ks < ke) GK_LOAD(ks, wc, xc)
     // (the rows' scales for the gated epilogue: formed by the last wave while its first loads are
     // on their way, handed to the first wave through LDS)
-    constexpr bool SCALES = EPI == EPI_SWIGLU && !PARTIAL;
+    constexpr bool SCALES = epi_gated(EPI) && !PARTIAL;
     __shared__ float gk_scale[16];
     __shared__ __attribute__((aligned(16))) float gk_red[SCALES ? 16 * RS_RED_STRIDE : 4];
     if (SCALES && wave == 3) {
@@ -733,12 +742,12 @@ gemm_kpar_kernel(const bf16_t* __restrict__ x, int ldx, const bf16_t* __restrict
     for (int e = 0; e < 4; ++e) sum[e] = ((red[0][lane][e] + red[1][lane][e]) + red[2][lane][e]) + red[3][lane][e];
     // element e of a lane: weight row 4g + e of the tile, activation row lane%16
     int gn0 = tile * 16 + g * 4;
-    if (EPI == EPI_SWIGLU && !PARTIAL) {
+    if (epi_gated(EPI) && !PARTIAL) {
 #pragma unroll
         for (int e = 0; e < 4; e += 2)
             if (gn0 + e + 1 < n)
                 ((bf16_t*)out)[(size_t)col * ldo + ((gn0 + e) >> 1)] =
-                    f32_to_bf16(silu_mul(sum[e] * row_scale, sum[e + 1] * row_scale));
+                    f32_to_bf16(gated_mul<EPI>(sum[e] * row_scale, sum[e + 1] * row_scale));
         return;
     }
 #pragma unroll

@@ -14,7 +14,13 @@ constexpr int GT_BM = 64, GT_BN = 64, GT_BK = 16, GT_THREADS = 256;
 template <typename TX, typename TW, typename TO, bool ACCUM>
 __global__ void __launch_bounds__(GT_THREADS)
 gemm_tile_kernel(const TX* __restrict__ x, int ldx, const TW* __restrict__ w, int ldw,
-                 TO* __restrict__ out, int ldo, int m, int n, int k) {
+                 TO* __restrict__ out, int ldo, int m, int n, int k,
+                 long long batch_x = 0, long long batch_w = 0, long long batch_o = 0) {
+    // blockIdx.z numbers the products of a batch: product b reads x + b * batch_x and
+    // w + b * batch_w and writes out + b * batch_o (one product per head of a layer, say).
+    x += (size_t)blockIdx.z * batch_x;
+    w += (size_t)blockIdx.z * batch_w;
+    out += (size_t)blockIdx.z * batch_o;
     __shared__ float xs[GT_BK][GT_BM + 4];
     __shared__ float ws[GT_BK][GT_BN + 4];
     int tid = threadIdx.x;
@@ -73,4 +79,15 @@ static void launch_gemm_tile(const void* x, int ldx, const void* w, int ldw, voi
     else
         gemm_tile_kernel<TX, TW, TO, false><<<grid, GT_THREADS, 0, stream>>>(
             (const TX*)x, ldx, (const TW*)w, ldw, (TO*)out, ldo, m, n, k);
+}
+
+// A batch of products of one shape: product b is out_b[M, N] = x_b[M, K] * w_b[N, K]^T with
+// x_b = x + b * batch_x (rows ldx apart), w_b = w + b * batch_w, out_b = out + b * batch_o.
+template <typename TX, typename TW, typename TO>
+static void launch_gemm_tile_batched(const void* x, int ldx, long long batch_x, const void* w, int ldw, long long batch_w,
+                                     void* out, int ldo, long long batch_o, int batch, int m, int n, int k,
+                                     hipStream_t stream) {
+    dim3 grid(ceil_div(n, GT_BN), ceil_div(m, GT_BM), batch);
+    gemm_tile_kernel<TX, TW, TO, false><<<grid, GT_THREADS, 0, stream>>>(
+        (const TX*)x, ldx, (const TW*)w, ldw, (TO*)out, ldo, m, n, k, batch_x, batch_w, batch_o);
 }

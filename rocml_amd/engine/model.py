@@ -9,6 +9,7 @@ from typing import Dict, List, Optional
 
 import torch
 
+from .. import ops
 from ..cache import Cache
 from ..cache.cache import HEADROOM_BYTES
 from ..config.spec import ModelSpec
@@ -39,6 +40,8 @@ class DecoderModel:
         self.embedding = build_embedding(spec.embedding_spec(), ctx)
         self.blocks = [build_block(b, ctx) for b in spec.layers]
         self.head = build_head(spec.head_spec(), ctx)
+        # rows that schedule entries add to the residual stream before they run (32-bit)
+        self.pass_offset: Optional[torch.Tensor] = None
         self.bound = False
         # whether a decode step may be recorded as a graph: every part must say so
         self.graph_safe = all(getattr(part, "graph_safe", True)
@@ -64,6 +67,8 @@ class DecoderModel:
         for i, block in enumerate(self.blocks):
             for name, p in block.param_specs().items():
                 specs[f"layers.{i}.{name}"] = p
+        if self.spec.pass_offsets:
+            specs["pass_offset.weight"] = ParamSpec((self.spec.pass_offsets, self.spec.hidden), role="gain", init="normal")
         specs.update(self.head.param_specs())
         return specs
 
@@ -76,6 +81,8 @@ class DecoderModel:
             prefix = f"layers.{i}."
             block.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
         self.head.bind({k: tensors[k] for k in self.head.param_specs()}, shared=self.embedding.shared_matrix())
+        if self.spec.pass_offsets:
+            self.pass_offset = tensors["pass_offset.weight"]
         self.bound = True
 
     def weight_bytes(self) -> int:
@@ -166,11 +173,16 @@ class DecoderModel:
                 group, line = cache.line(owner)
                 view = group.view(line, step)
             block = self.blocks[entry.layer]
+            if entry.offset_row is not None:
+                # (sums that a product left for the next norm may still be missing from x: additions commute)
+                ops.add_row_vector(x, self.pass_offset[entry.offset_row])
             if not getattr(block, "takes_pending", False):
                 ws.flush_pending()
             # the block that runs next may let this block's last product prepare its first norm
             following = self.blocks[s.schedule[i + 1].layer] if i + 1 < len(s.schedule) else None
             hint = None
+            if following is not None and s.schedule[i + 1].offset_row is not None:
+                following = None      # the stream changes between the two blocks: nothing can be prepared across
             if getattr(block, "takes_next_norm", False) and hasattr(following, "entry_hint"):
                 hint = following.entry_hint(step)
             if hint is not None:

@@ -29,21 +29,26 @@ _SIGNATURES = {
     "elementwise": {
         "rocml_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _F, _P],
         "rocml_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P, _I, _LL, _P],
-        "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _I, _P],
+        "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _I, _I, _P],
         "rocml_rope_table": [_P, _P, _P, _P, _I, _I, _P],
         "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _I, _P, _P, _P,
-                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P],
+                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _P],
         "rocml_add_into": [_P, _P, _I, _LL, _P],
+        "rocml_add_row_vector": [_P, _P, _I, _I, _P],
+        "rocml_latent_prepare": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _P],
+        "rocml_rope_heads": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+        "rocml_sigmoid_gate": [_P, _I, _P, _I, _I, _I, _P],
     },
     "gemm": {
         "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _LL, _P, _I, _F, _I, _P],
         "rocml_splitk_reduce": [_P, _P, _I, _I, _I, _I, _I, _I, _P],
+        "rocml_gemm_batched": [_P, _I, _I, _LL, _P, _I, _I, _LL, _P, _I, _I, _LL, _I, _I, _I, _I, _P],
         "rocml_gemm_residual_prescale_pays": [_I, _I, _I],
         "rocml_gemm_residual_prescale": [_P, _I, _P, _I, _P, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P],
     },
     "attention": {
         "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
-                            _P, _I, _I, _P, _I, _I, _P, _LL, _P],
+                            _P, _I, _I, _P, _I, _I, _P, _LL, _I, _I, _I, _P, _I, _P],
         "rocml_attention_decode_fused": [_P, _I, _I, _LL, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P,
                                          _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P, _I, _F, _I, _P],
         "rocml_attention_prefill_fused": [_P, _I, _P, _F, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I,
@@ -190,15 +195,21 @@ def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
         stride, _stream()))
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool = False) -> None:
-    """``gate_up`` rows hold the gate half then the up half, or (gate, up) pairs when
-    ``interleaved``."""
+GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool = False, activation: str = "silu") -> None:
+    """``out = act(gate) * up``.  ``gate_up`` rows hold the gate half then the up half, or (gate, up)
+    pairs when ``interleaved``; ``activation`` is one of ``GATE_ACTIVATIONS``."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"unknown activation {activation!r}; known: {sorted(GATE_ACTIVATIONS)}")
     _dev(gate_up, out)
     n_tokens, inter = out.shape
     if gate_up.shape != (n_tokens, 2 * inter):
         raise KernelError(f"gate/up is {tuple(gate_up.shape)}, expected {(n_tokens, 2 * inter)}")
     _check("elementwise", library("elementwise").rocml_swiglu(
-        _ptr(gate_up), _code(gate_up), _ptr(out), _code(out), n_tokens, inter, 1 if interleaved else 0, _stream()))
+        _ptr(gate_up), _code(gate_up), _ptr(out), _code(out), n_tokens, inter, 1 if interleaved else 0,
+        GATE_ACTIVATIONS[activation], _stream()))
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
@@ -223,16 +234,21 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
                         q_out: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                         v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                         token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True,
-                        n_splits: int = 1, pairing: str = "halves") -> None:
+                        n_splits: int = 1, pairing: str = "halves", bias: Optional[torch.Tensor] = None,
+                        v_head_dim: Optional[int] = None) -> None:
     """``qkv`` is ``[T, ld]`` with q, k, v side by side (k and v may be absent when
     ``write_kv`` is false).  Keys are ``[pages, Hkv, page_size, D]``, values
     ``[pages, Hkv, D, page_size]``.  ``pairing``: which two values of the rotated width turn
     together by the angle in column ``i`` of the tables: ``"halves"``, ``(i, i + rot_dim / 2)``,
     or ``"neighbours"``, ``(2 i, 2 i + 1)``.  ``q_out`` None: only keys and values are prepared
-    and appended (the caller's attention kernel prepares its queries itself)."""
+    and appended (the caller's attention kernel prepares its queries itself).  ``bias``: 32-bit,
+    one number per column of ``qkv``, added to the projection's sums.  ``v_head_dim``: the size of a
+    value head when it is not ``head_dim`` (the value columns then follow the ``Hq + Hkv`` heads of
+    ``head_dim``)."""
+    dv = head_dim if v_head_dim is None else int(v_head_dim)
     if pairing not in ROPE_PAIRINGS:
         raise KernelError(f"unknown rotation pairing {pairing!r}; known: {sorted(ROPE_PAIRINGS)}")
-    _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos)
+    _dev(qkv, q_gain, k_gain, cos, sin, q_out, k_cache, v_cache, block_table, token_seq, token_pos, bias)
     split_stride = 0
     if n_splits > 1:                      # [splits, T, ld] split-K partial sums, added in the kernel
         if qkv.dim() != 3 or qkv.shape[0] != n_splits:
@@ -240,6 +256,10 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         split_stride = qkv.shape[1] * qkv.shape[2]
         qkv = qkv[0]
     n_tokens, ld = qkv.shape
+    if bias is not None:
+        _want(bias, torch.float32, "projection bias")
+        if bias.numel() != ld:
+            raise KernelError(f"the bias has {bias.numel()} values for rows of {ld}")
     for g in (q_gain, k_gain):
         if g is not None:
             _want(g, torch.float32, "head norm gain")
@@ -258,7 +278,7 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         if k_cache is None or v_cache is None or block_table is None:
             raise KernelError("appending to the cache needs the cache and the block table")
         if k_cache.shape[1:] != (n_kv_heads, k_cache.shape[2], head_dim) \
-                or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, k_cache.shape[2]):
+                or v_cache.shape != (k_cache.shape[0], n_kv_heads, dv, k_cache.shape[2]):
             raise KernelError(f"cache shape {tuple(k_cache.shape)} does not fit {n_kv_heads} heads of {head_dim}")
         if q_out is not None and k_cache.dtype != q_out.dtype:
             raise KernelError("cache and q output must share their type")
@@ -268,7 +288,89 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         _ptr(qkv), _code(qkv), ld, n_tokens, n_heads, n_kv_heads, head_dim, _ptr(q_gain), _ptr(k_gain),
         eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, ROPE_PAIRINGS[pairing], _ptr(q_out), _ptr(k_cache),
         _ptr(v_cache), _code(q_out if q_out is not None else k_cache), _ptr(block_table), bt_width, _ptr(token_seq),
-        _ptr(token_pos), page_size, 1 if write_kv else 0, n_splits, split_stride, _stream()))
+        _ptr(token_pos), page_size, 1 if write_kv else 0, n_splits, split_stride, _ptr(bias), dv, _stream()))
+
+
+def add_row_vector(x: torch.Tensor, b: torch.Tensor) -> None:
+    """``x[t, :] += b`` for the 32-bit ``x [T, n]`` and ``b [n]``."""
+    _dev(x, b)
+    _want(x, torch.float32, "residual stream")
+    _want(b, torch.float32, "row vector")
+    if x.dim() != 2 or b.numel() != x.shape[1]:
+        raise KernelError(f"a vector of {b.numel()} numbers does not fit rows of {tuple(x.shape)}")
+    _check("elementwise", library("elementwise").rocml_add_row_vector(_ptr(x), _ptr(b), x.shape[0], x.shape[1], _stream()))
+
+
+def latent_prepare(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_part: int, rot_dims: int,
+                   q_gain: torch.Tensor, kv_gain: torch.Tensor, eps: float, cos: Optional[torch.Tensor],
+                   sin: Optional[torch.Tensor], cq_out: torch.Tensor, cache: Optional[torch.Tensor],
+                   block_table: Optional[torch.Tensor], token_seq: torch.Tensor, token_pos: torch.Tensor,
+                   write_cache: bool = True) -> None:
+    """What follows a latent attention's first projection.  A row of ``proj`` (32-bit) holds the
+    query latent (``q_rank``), the key/value latent (``kv_rank``) and the shared rotated key part
+    (``rot_part``, of which the first ``rot_dims`` turn in pairs ``(i, i + rot_dims/2)``).  Both
+    latents get their root-mean-square norm; the query latent goes to ``cq_out [T, q_rank]``, the
+    other two into the token's row of ``cache [pages, page_size, kv_rank + rot_part]``."""
+    _dev(proj, q_gain, kv_gain, cos, sin, cq_out, cache, block_table, token_seq, token_pos)
+    _want(proj, torch.float32, "projection output")
+    _want(q_gain, torch.float32, "latent norm gain")
+    _want(kv_gain, torch.float32, "latent norm gain")
+    n_tokens, ld = proj.shape
+    if q_gain.numel() != q_rank or kv_gain.numel() != kv_rank or cq_out.shape != (n_tokens, q_rank):
+        raise KernelError("latent gains or the query latent's output do not fit the ranks")
+    if rot_dims:
+        if cos is None or sin is None or cos.shape != (n_tokens, rot_dims // 2) or sin.shape != cos.shape \
+                or cos.dtype != torch.float32 or sin.dtype != torch.float32:
+            raise KernelError(f"rotation tables must be float32 {(n_tokens, rot_dims // 2)}")
+    page_size = bt_width = 0
+    if write_cache:
+        if cache is None or block_table is None:
+            raise KernelError("appending to the cache needs the cache and the block table")
+        if cache.dim() != 3 or cache.shape[2] != kv_rank + rot_part or cache.dtype != cq_out.dtype:
+            raise KernelError(f"latent cache {tuple(cache.shape)} {cache.dtype} does not fit rows of {kv_rank + rot_part}")
+        _want(block_table, torch.int32, "block table")
+        page_size, bt_width = cache.shape[1], block_table.shape[1]
+    _want(token_seq, torch.int32, "token sequence table")
+    _want(token_pos, torch.int32, "token position table")
+    if token_seq.numel() != n_tokens or token_pos.numel() != n_tokens:
+        raise KernelError("one sequence index and one position per token are needed")
+    _check("elementwise", library("elementwise").rocml_latent_prepare(
+        _ptr(proj), ld, n_tokens, q_rank, kv_rank, rot_part, rot_dims, _ptr(q_gain), _ptr(kv_gain), eps, _ptr(cos),
+        _ptr(sin), _ptr(cq_out), _ptr(cache), _code(cq_out), _ptr(block_table), bt_width, _ptr(token_seq),
+        _ptr(token_pos), page_size, 1 if write_cache else 0, _stream()))
+
+
+def rope_heads(q: torch.Tensor, n_heads: int, head_stride: int, offset: int, rot_part: int, rot_dims: int,
+               cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], out: torch.Tensor, out_stride: int,
+               out_offset: int) -> None:
+    """The part of every head of ``q [T, n_heads * head_stride]`` (32-bit) that starts at ``offset``
+    and is ``rot_part`` wide, rotated (its first ``rot_dims`` numbers, pairs ``(i, i + rot_dims/2)``),
+    written to ``out [T, n_heads * out_stride]`` at ``out_offset`` of every head."""
+    _dev(q, cos, sin, out)
+    _want(q, torch.float32, "queries")
+    n_tokens = q.shape[0]
+    if q.dim() != 2 or out.dim() != 2 or out.shape[0] != n_tokens:
+        raise KernelError("queries and output must be [tokens, width]")
+    if rot_dims and (cos is None or sin is None or cos.shape != (n_tokens, rot_dims // 2) or sin.shape != cos.shape
+                     or cos.dtype != torch.float32 or sin.dtype != torch.float32):
+        raise KernelError(f"rotation tables must be float32 {(n_tokens, rot_dims // 2)}")
+    _check("elementwise", library("elementwise").rocml_rope_heads(
+        _ptr(q), q.shape[1], head_stride, offset, rot_part, rot_dims, _ptr(cos), _ptr(sin), _ptr(out), _code(out),
+        out.shape[1], out_stride, out_offset, n_tokens, n_heads, _stream()))
+
+
+def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> None:
+    """``y *= sigmoid(gate)`` for ``y [T, n]`` and the 32-bit ``gate [T, n]``, whose rows may be a
+    column range of a wider matrix."""
+    _dev(y)
+    if not gate.is_cuda:
+        raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
+    _want(gate, torch.float32, "gate")
+    if y.dim() != 2 or gate.shape != y.shape or gate.stride(1) != 1:
+        raise KernelError(f"gate {tuple(gate.shape)} does not fit {tuple(y.shape)}")
+    ldg = gate.stride(0) if y.shape[0] > 1 else max(gate.stride(0), y.shape[1])
+    _check("elementwise", library("elementwise").rocml_sigmoid_gate(_ptr(y), _code(y), _ptr(gate), ldg, y.shape[0],
+                                                                   y.shape[1], _stream()))
 
 
 def add_into(x: torch.Tensor, y: torch.Tensor) -> None:
@@ -281,6 +383,8 @@ def add_into(x: torch.Tensor, y: torch.Tensor) -> None:
 
 # ---- matrix product ------------------------------------------------------------------
 GEMM_AUTO, GEMM_PLAIN = 0, 1
+# epilogues of a product whose weight rows are (gate, up) pairs: act(gate) * up
+GEMM_EPILOGUES = {None: 0, "swiglu": 1, "relu_glu": 2}
 ROW_SCALE_MAX_ROWS = 16     # most rows of a product whose consumer applies a row scale
 
 
@@ -314,7 +418,7 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
             raise KernelError("kernel arguments must be GPU tensors; this library has no CPU path")
         if t.dim() != 2 or t.stride(1) != 1:
             raise KernelError("matrix product operands must be 2-D with unit inner stride")
-    if epilogue not in (None, "swiglu"):
+    if epilogue not in GEMM_EPILOGUES:
         raise KernelError(f"unknown epilogue {epilogue!r}")
     m, k = x.shape
     n = w.shape[0]
@@ -325,15 +429,30 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     deferred = ctypes.c_int(0)
     ssq_ptr, parts, eps = None, 0, 0.0
     if row_scale is not None:
-        if epilogue != "swiglu" or m > ROW_SCALE_MAX_ROWS or row_scale.width != k or row_scale.ssq.shape[0] < m:
+        if epilogue is None or m > ROW_SCALE_MAX_ROWS or row_scale.width != k or row_scale.ssq.shape[0] < m:
             raise KernelError("a row scale goes with the gated epilogue of at most 16 rows whose K is the norm's width")
         ssq_ptr, parts, eps = row_scale.ssq.data_ptr(), row_scale.ssq.shape[1], row_scale.eps
     _check("gemm", library("gemm").rocml_gemm(
         _ptr(x), _code(x), x.stride(0) if m > 1 else max(x.stride(0), k), _ptr(w), _code(w), w.stride(0),
         _ptr(out), _code(out), out.stride(0) if m > 1 else max(out.stride(0), cols), m, n, k,
-        1 if accumulate else 0, algo, 1 if epilogue else 0, 1 if defer else 0, ctypes.byref(deferred), ws_ptr,
+        1 if accumulate else 0, algo, GEMM_EPILOGUES[epilogue], 1 if defer else 0, ctypes.byref(deferred), ws_ptr,
         ws_bytes, ssq_ptr, parts, eps, int(max_splits), _stream()))
     return deferred.value
+
+
+def gemm_batched(x: torch.Tensor, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_head_stride: int) -> None:
+    """One small product per head: ``out[:, h * out_head_stride : ... + N] = x[:, h * x_head_stride :
+    ... + K] @ w[h].T`` for ``w [heads, N, K]``; ``x`` and ``out`` are ``[tokens, width]`` matrices
+    that hold the heads side by side.  32-bit accumulation; ``x`` may be 32-bit with bfloat16 weights."""
+    _dev(x, w, out)
+    if x.dim() != 2 or out.dim() != 2 or w.dim() != 3 or x.shape[0] != out.shape[0]:
+        raise KernelError("gemm_batched takes x [T, width], w [heads, N, K], out [T, width]")
+    heads, n, k = w.shape
+    if (heads - 1) * x_head_stride + k > x.shape[1] or (heads - 1) * out_head_stride + n > out.shape[1]:
+        raise KernelError(f"{heads} heads of K={k} / N={n} do not fit rows of {x.shape[1]} / {out.shape[1]}")
+    _check("gemm", library("gemm").rocml_gemm_batched(
+        _ptr(x), _code(x), x.shape[1], x_head_stride, _ptr(w), _code(w), k, n * k, _ptr(out), _code(out),
+        out.shape[1], out_head_stride, heads, x.shape[0], n, k, _stream()))
 
 
 PRESCALE_MAX_ROWS = 16      # most rows gemm_residual_prescale takes
@@ -401,20 +520,39 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
               n_heads: int, n_kv_heads: int, head_dim: int, scale: float, window: Optional[int] = None,
               algo: int = ATTN_AUTO, workspace: Optional[torch.Tensor] = None,
               cu_seqlens: Optional[torch.Tensor] = None, max_new: int = 0,
-              q_counts: Optional[Sequence[int]] = None, max_len: int = 0, n_splits: int = 0) -> None:
+              q_counts: Optional[Sequence[int]] = None, max_len: int = 0, n_splits: int = 0,
+              v_head_dim: Optional[int] = None, values_in_keys: bool = False, chunk: Optional[int] = None,
+              slopes: Optional[torch.Tensor] = None, sink: bool = False) -> None:
     """Attention of the step's query tokens over the cache.  Keys are ``[pages, Hkv, page, D]``,
     values ``[pages, Hkv, D, page]``.  ``cu_seqlens`` (device), ``q_counts`` (the same knowledge on
     the host: query tokens of each sequence), ``max_new`` (the most of them) and ``max_len``
-    (longest context) describe the step to the fast kernels; without them the plain kernel runs."""
-    _dev(q, out, k_cache, v_cache, block_table, token_seq, token_pos, cu_seqlens)
+    (longest context) describe the step to the fast kernels; without them the plain kernel runs.
+
+    ``v_head_dim``: size of a value head when it is not ``head_dim``.  ``values_in_keys``: there is
+    no value cache (``v_cache`` None) and a key's value is the first ``v_head_dim`` numbers of its
+    row.  ``chunk``: blocks of so many positions, counted from 0, instead of a window: a query sees
+    its own block up to itself.  ``slopes`` (32-bit, one per query head): ``slope * (i - j)`` is
+    taken off the score of query ``i`` and key ``j``.  ``sink``: the denominator of the softmax has
+    one more term ``exp(0)``."""
+    _dev(q, out, k_cache, v_cache, block_table, token_seq, token_pos, cu_seqlens, slopes)
     n_tokens = q.shape[0]
-    if q.shape != (n_tokens, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype:
-        raise KernelError("attention input and output must both be [tokens, heads * head_dim] of one type")
+    dv = head_dim if v_head_dim is None else int(v_head_dim)
+    if q.shape != (n_tokens, n_heads * head_dim) or out.shape != (n_tokens, n_heads * dv) or out.dtype != q.dtype:
+        raise KernelError("attention input must be [tokens, heads * head_dim] and its output [tokens, heads * value size], of one type")
     page = k_cache.shape[2]
-    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype \
-            or k_cache.shape[1:] != (n_kv_heads, page, head_dim) \
-            or v_cache.shape != (k_cache.shape[0], n_kv_heads, head_dim, page):
-        raise KernelError(f"cache {tuple(k_cache.shape)} / {tuple(v_cache.shape)} {k_cache.dtype} does not fit the queries")
+    if k_cache.dtype != q.dtype or k_cache.shape[1:] != (n_kv_heads, page, head_dim):
+        raise KernelError(f"key cache {tuple(k_cache.shape)} {k_cache.dtype} does not fit the queries")
+    if values_in_keys:
+        if v_cache is not None or dv > head_dim:
+            raise KernelError("values taken from the key rows: no value cache, and a value no longer than a key")
+    elif v_cache is None or v_cache.dtype != q.dtype or v_cache.shape != (k_cache.shape[0], n_kv_heads, dv, page):
+        raise KernelError(f"value cache does not fit keys {tuple(k_cache.shape)} and a value size of {dv}")
+    if slopes is not None:
+        _want(slopes, torch.float32, "distance slopes")
+        if slopes.numel() != n_heads:
+            raise KernelError("one distance slope per query head is needed")
+    if chunk is not None and window is not None:
+        raise KernelError("a layer has a window or blocks of positions, not both")
     _want(block_table, torch.int32, "block table")
     _want(token_seq, torch.int32, "token sequence table")
     _want(token_pos, torch.int32, "token position table")
@@ -434,7 +572,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache
         _ptr(q), _ptr(out), _ptr(k_cache), _ptr(v_cache), _code(q), _ptr(block_table),
         block_table.shape[1], _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim,
         page, scale, 0 if window is None else int(window), algo, _ptr(cu_seqlens), n_seqs, max_new,
-        counts, max_len, n_splits, ws_ptr, ws_bytes, _stream()))
+        counts, max_len, n_splits, ws_ptr, ws_bytes, dv, 1 if values_in_keys else 0,
+        0 if chunk is None else int(chunk), _ptr(slopes), 1 if sink else 0, _stream()))
 
 
 FUSED_DECODE_HEAD_DIMS = (64, 128, 192, 256)

@@ -7,6 +7,12 @@ Here q, k and v come from one product over the concatenated weight, norm + rotat
 append are one kernel, and the residual sum is the output product's epilogue.  Head
 counts, head size, scale, window, the optional norm and the optional position encoding
 are the spec's, nothing is fixed here.
+
+A layer may also ask for biased projections, a value head of another size than the key head,
+blocks of positions instead of a window, a penalty on distance (a slope per head) and a sink in
+the softmax.  Any of these takes the layer off the matrix-core attention kernels, which know none
+of them, and onto the plain kernel, which takes them all as parameters; the projections and the
+append kernel are the same ones.
 """
 from __future__ import annotations
 
@@ -36,11 +42,24 @@ class Attention(Mixer):
             raise ConfigError(f"the per-head norm must be of kind 'rmsnorm', got {spec.qk_norm.kind!r}")
         if spec.window is not None and spec.window <= 0:
             raise ConfigError(f"window must be positive, got {spec.window}")
+        if spec.chunk is not None and (spec.chunk <= 0 or spec.window is not None):
+            raise ConfigError("blocks of positions must be positive in size and exclude a window")
+        if spec.distance_slopes is not None and len(spec.distance_slopes) != spec.n_heads:
+            raise ConfigError(f"{len(spec.distance_slopes)} distance slopes for {spec.n_heads} heads")
+        self.v_head_dim = spec.head_dim if spec.v_head_dim is None else spec.v_head_dim
+        # what the matrix-core kernels do not know: such a layer runs the plain attention kernel
+        self.extras = (self.v_head_dim != spec.head_dim or spec.chunk is not None
+                       or spec.distance_slopes is not None or spec.sink)
+        self.slopes: Optional[torch.Tensor] = None
+        if spec.distance_slopes is not None and torch.device(ctx.device).type != "meta":
+            self.slopes = torch.tensor(spec.distance_slopes, dtype=torch.float32, device=ctx.device)
         self.spec = spec
         self.dtype = ctx.dtype
         self.n_cus = ops.cu_count(ctx.device)
         self.q_dim = spec.n_heads * spec.head_dim
         self.kv_dim = spec.n_kv_heads * spec.head_dim
+        self.v_dim = spec.n_kv_heads * self.v_head_dim
+        self.o_dim = spec.n_heads * self.v_head_dim
         self.position = build_position(spec.position, ctx) if spec.position is not None else None
         self.pairing = getattr(self.position, "pairing", "halves")
         if self.pairing not in ops.ROPE_PAIRINGS:
@@ -53,13 +72,20 @@ class Attention(Mixer):
         self.w_o: Optional[torch.Tensor] = None
         self.q_gain: Optional[torch.Tensor] = None
         self.k_gain: Optional[torch.Tensor] = None
+        self.b_qkv: Optional[torch.Tensor] = None
+        self.b_o: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         s = self.spec
         specs = {"q_proj.weight": ParamSpec((self.q_dim, s.hidden)),
                  "k_proj.weight": ParamSpec((self.kv_dim, s.hidden)),
-                 "v_proj.weight": ParamSpec((self.kv_dim, s.hidden)),
-                 "o_proj.weight": ParamSpec((s.hidden, self.q_dim))}
+                 "v_proj.weight": ParamSpec((self.v_dim, s.hidden)),
+                 "o_proj.weight": ParamSpec((s.hidden, self.o_dim))}
+        if s.bias:       # added in 32-bit to the products' sums
+            specs.update({"q_proj.bias": ParamSpec((self.q_dim,), role="gain", init="normal"),
+                          "k_proj.bias": ParamSpec((self.kv_dim,), role="gain", init="normal"),
+                          "v_proj.bias": ParamSpec((self.v_dim,), role="gain", init="normal"),
+                          "o_proj.bias": ParamSpec((s.hidden,), role="gain", init="normal")})
         if s.qk_norm is not None:
             specs["q_norm.weight"] = ParamSpec((s.head_dim,), role="gain", init="gain")
             specs["k_norm.weight"] = ParamSpec((s.head_dim,), role="gain", init="gain")
@@ -71,6 +97,9 @@ class Attention(Mixer):
         self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
                                 tensors["v_proj.weight"]], dim=0).contiguous()
         self.w_o = tensors["o_proj.weight"]
+        if self.spec.bias:
+            self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]).contiguous()
+            self.b_o = tensors["o_proj.bias"]
         if self.spec.qk_norm is not None:
             self.q_gain = tensors["q_norm.weight"]
             self.k_gain = tensors["k_norm.weight"]
@@ -78,22 +107,25 @@ class Attention(Mixer):
     def flops(self, new_counts, starts) -> int:
         # the products with the weights, and 4 * heads * head size per query and key it sees
         keys = 0
-        w = self.spec.window
+        w, c = self.spec.window, self.spec.chunk
         for n, s0 in zip(new_counts, starts):
-            if w is None:
+            if c is not None:
+                keys += sum((s0 + i) % c + 1 for i in range(n))
+            elif w is None:
                 keys += n * s0 + n * (n + 1) // 2
             else:
                 keys += sum(min(s0 + i + 1, w) for i in range(n))
-        return 2 * sum(new_counts) * self.matrix_elements() + 4 * self.spec.n_heads * self.spec.head_dim * keys
+        return 2 * sum(new_counts) * self.matrix_elements() + \
+            2 * self.spec.n_heads * (self.spec.head_dim + self.v_head_dim) * keys
 
     def activation_bytes(self, n_tokens: int) -> int:
         size = 2 if self.dtype == torch.bfloat16 else 4
         rot = 0 if self.position is None else 2 * n_tokens * (self.position.rot_dim // 2) * 4
-        return n_tokens * ((self.q_dim + 2 * self.kv_dim) * 4 + 2 * self.q_dim * size) + rot
+        return n_tokens * ((self.q_dim + self.kv_dim + self.v_dim) * 4 + (self.q_dim + self.o_dim) * size) + rot
 
     def _fused_decode(self, step) -> bool:
         rot = None if self.position is None else self.position.rot_dim
-        return step.max_new == 1 and ops.attention_decode_fusable(
+        return not self.extras and not self.spec.bias and step.max_new == 1 and ops.attention_decode_fusable(
             self.dtype, self.spec.n_heads, self.spec.n_kv_heads, self.spec.head_dim, ops.FUSED_DECODE_PAGE, rot, self.pairing)
 
     def _fused_prefill(self, step, cache) -> bool:
@@ -101,7 +133,7 @@ class Attention(Mixer):
         tokens on (the preparation lengthens every attention block by some 6 us, the norm-and-rotation
         kernel's q rows cost 8 us per thousand tokens at 32 heads of 128)."""
         rot = None if self.position is None else self.position.rot_dim
-        return (step.max_new > 1 and step.n_tokens >= self.FUSED_PREFILL_MIN_TOKENS
+        return (not self.extras and not self.spec.bias and step.max_new > 1 and step.n_tokens >= self.FUSED_PREFILL_MIN_TOKENS
                 and step.cu_seqlens is not None and self.dtype == torch.bfloat16
                 and ops.attention_prefill_fusable(cache.k.dtype, self.spec.head_dim, cache.k.shape[2], rot, self.pairing))
 
@@ -110,7 +142,10 @@ class Attention(Mixer):
         return self._fused_decode(step)
 
     def cache_request(self) -> KVCacheRequest:
-        return KVCacheRequest(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
+        s = self.spec
+        if s.v_head_dim is None and s.chunk is None:
+            return KVCacheRequest(s.n_kv_heads, s.head_dim, s.window)
+        return KVCacheRequest(s.n_kv_heads, s.head_dim, s.window, v_head_dim=self.v_head_dim, chunk=s.chunk)
 
     def _decode_splits(self, step, cache) -> int:
         """Splits of the key range in a decode step: enough blocks to fill the chip, at most one
@@ -124,7 +159,7 @@ class Attention(Mixer):
         s = self.spec
         n = step.n_tokens
         ws = step.workspace
-        rows = self.q_dim + 2 * self.kv_dim if owns_cache else self.q_dim
+        rows = self.q_dim + self.kv_dim + self.v_dim if owns_cache else self.q_dim
         qkv = ws.get("attn.qkv", (n, rows), torch.float32)
         scratch = ws.scratch()
         # (the decode kernel that reads the projection adds four partial sums in one trip to memory
@@ -139,7 +174,7 @@ class Attention(Mixer):
             cos, sin = self.position.tables(step)
             rot = self.position.rot_dim
         eps = s.qk_norm.eps if s.qk_norm is not None else 1.0
-        o = ws.get("attn.o", (n, self.q_dim), self.dtype)
+        o = ws.get("attn.o", (n, self.o_dim), self.dtype)
         if self._fused_decode(step) and cache.k.dtype == self.dtype and cache.k.shape[2] == ops.FUSED_DECODE_PAGE:
             # One token per sequence: norm, rotation, append and attention in one launch, straight
             # from the projection.  The attention's own partial results go behind the projection's.
@@ -165,13 +200,19 @@ class Attention(Mixer):
                                             step.cu_seqlens, step.new_counts, max_len=step.max_len)
             else:
                 q = ws.get("attn.q", (n, self.q_dim), self.dtype)
+                bias = None if self.b_qkv is None else self.b_qkv[:rows]
                 ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
                                         cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
-                                        step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1), pairing=self.pairing)
+                                        step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1), pairing=self.pairing,
+                                        bias=bias, v_head_dim=self.v_head_dim)
                 ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
                               s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                               cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
-                              max_len=step.max_len, n_splits=self._decode_splits(step, cache))
+                              max_len=step.max_len, n_splits=self._decode_splits(step, cache),
+                              v_head_dim=self.v_head_dim, chunk=s.chunk, slopes=self.slopes, sink=s.sink)
+        if self.b_o is not None:
+            ws.flush_pending()
+            ops.add_row_vector(x_accum, self.b_o)
         stream(step).add_product(o, self.w_o, x_accum)
 
 

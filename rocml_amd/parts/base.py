@@ -39,7 +39,8 @@ class ParamSpec:
     ``gain``: a small vector used in 32-bit arithmetic, always held in 32-bit.
     ``int_table``: integers, held as int32.
     ``init`` names how random weights are drawn: ``normal`` is N(0, 0.02), ``gain`` is 1
-    (or 1 + N(0, 0.02) when jitter is asked for), ``zeros`` is 0."""
+    (or 1 + N(0, 0.02) when jitter is asked for), ``offset`` is 0 (or N(0, 0.02) with jitter: a
+    gain stored as its distance from one), ``zeros`` is 0."""
     shape: Tuple[int, ...]
     role: str = "matrix"
     init: str = "normal"
@@ -53,10 +54,24 @@ class BuildContext:
 
 @dataclass(frozen=True)
 class KVCacheRequest:
-    """Keys and values per position: ``window`` is None when all positions are kept."""
+    """Keys and values per position: ``window`` is None when all positions are kept.
+    ``v_head_dim``: size of a value head when it is not ``head_dim``.  ``chunk``: positions are
+    cut into blocks of so many, counted from 0, and no query looks back beyond the start of its
+    own block (so earlier blocks' pages can be given back)."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+    chunk: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class LatentCacheRequest:
+    """One row of ``width`` numbers per position (a latent from which keys and values are
+    expanded, and whatever key part is stored beside it); ``window`` as above."""
+    width: int
+    window: Optional[int] = None
+    chunk: Optional[int] = None
 
 
 @dataclass(frozen=True)

@@ -20,13 +20,14 @@ class PreNormBlock(Part):
         self.dtype = ctx.dtype
         self.hidden = spec.mixer_norm.size
         self.children = {"mixer_norm": build_norm(spec.mixer_norm, ctx),
-                         "mixer": build_mixer(spec.mixer, ctx),
-                         "ffn_norm": build_norm(spec.ffn_norm, ctx),
-                         "ffn": build_feed_forward(spec.ffn, ctx)}
+                         "mixer": build_mixer(spec.mixer, ctx)}
+        if spec.ffn is not None:          # a layer may be its mixer alone
+            self.children["ffn_norm"] = build_norm(spec.ffn_norm, ctx)
+            self.children["ffn"] = build_feed_forward(spec.ffn, ctx)
         self.mixer_norm = self.children["mixer_norm"]
         self.mixer = self.children["mixer"]
-        self.ffn_norm = self.children["ffn_norm"]
-        self.ffn = self.children["ffn"]
+        self.ffn_norm = self.children.get("ffn_norm")
+        self.ffn = self.children.get("ffn")
         self.graph_safe = all(getattr(c, "graph_safe", True) for c in self.children.values())
         self.prompt_graph_safe = all(getattr(c, "prompt_graph_safe", False) for c in self.children.values())
 
@@ -43,11 +44,12 @@ class PreNormBlock(Part):
         return self.mixer.cache_request()
 
     def flops(self, new_counts, starts) -> int:
-        return self.mixer.flops(new_counts, starts) + self.ffn.flops(new_counts, starts)
+        return self.mixer.flops(new_counts, starts) + (self.ffn.flops(new_counts, starts) if self.ffn is not None else 0)
 
     def activation_bytes(self, n_tokens: int) -> int:
         size = 2 if self.dtype == torch.bfloat16 else 4
-        return n_tokens * self.hidden * size + self.mixer.activation_bytes(n_tokens) + self.ffn.activation_bytes(n_tokens)
+        return n_tokens * self.hidden * size + self.mixer.activation_bytes(n_tokens) + \
+            (self.ffn.activation_bytes(n_tokens) if self.ffn is not None else 0)
 
     takes_pending = True      # forward() may be handed a stream that still lacks deferred sums
     takes_next_norm = True    # forward() accepts the hint of the norm that reads the stream after it
@@ -65,9 +67,12 @@ class PreNormBlock(Part):
         xn, rs.row_scale = self._norm(step, self.mixer_norm, x)
         if not getattr(self.mixer, "adds_only", False):
             ws.flush_pending()
-        rs.next_norm = self._hint(step, self.ffn_norm, self.ffn)
+        rs.next_norm = self._hint(step, self.ffn_norm, self.ffn) if self.ffn is not None else next_norm
         self.mixer.forward(step, xn, x, cache, owns_cache)
         rs.next_norm = None
+        if self.ffn is None:
+            rs.row_scale = None
+            return
         xn, rs.row_scale = self._norm(step, self.ffn_norm, x)
         if not getattr(self.ffn, "adds_only", False):
             ws.flush_pending()

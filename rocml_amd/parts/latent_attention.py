@@ -1,0 +1,149 @@
+"""Softmax attention whose keys and values are expanded from one small latent vector per position.
+
+Per token the layer projects its input ``h`` to a query latent ``c_q = norm(W_dq h)``, a
+key/value latent ``c = norm(W_dkv h)[:kv_rank]`` and one rotated key part ``k_r`` that all heads
+share; head ``a`` then has ``q_a = W_uq,a c_q = [q_a^n, q_a^r]`` (the second part rotated),
+``k_a(j) = [W_uk,a c_j, k_r(j)]`` and ``v_a(j) = W_uv,a c_j``.  The cache holds ``[c_j, k_r(j)]``
+and nothing per head.  The attention never expands the keys: since
+
+    q_a^n . (W_uk,a c_j) = (W_uk,a^T q_a^n) . c_j        and
+    sum_j p_j W_uv,a c_j = W_uv,a (sum_j p_j c_j),
+
+every head asks one shared key/value "head" whose keys are the cache rows ``[c_j, k_r(j)]`` and
+whose values are the first ``kv_rank`` numbers of the same rows, with the query
+``[W_uk,a^T q_a^n, q_a^r]``; the head's output is ``W_uv,a`` times what the attention returns.
+Both small products run once per token and head, whatever the number of keys.
+
+Launches of a step: one product for the three projections of ``h`` (query latent, key/value
+latent with its rotated part, output gate), one kernel that norms both latents, rotates and
+appends to the cache, the product ``W_uq``, the rotation of the queries' rotated parts, the
+per-head products with ``W_uk^T``, the attention, the per-head products with ``W_uv``, the gate,
+and the output product whose epilogue is the residual sum.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from ..config.spec import LatentAttentionSpec
+from ..errors import ConfigError
+from .base import BuildContext, LatentCacheRequest, Mixer, ParamSpec
+from .registry import build_position, register_mixer
+from .residual import stream
+
+
+class LatentAttention(Mixer):
+    adds_only = True
+
+    def __init__(self, spec: LatentAttentionSpec, ctx: BuildContext):
+        for norm in (spec.q_norm, spec.kv_norm):
+            if norm.kind != "rmsnorm" or getattr(norm, "unit_offset", False):
+                # the latents are normed inside the kernel that appends to the cache, which knows one kind
+                raise ConfigError("the latents' norms must be plain root-mean-square norms")
+        if spec.q_norm.size != spec.q_rank or spec.kv_norm.size != spec.kv_rank:
+            raise ConfigError("the latents' norms must span the latents")
+        if spec.q_norm.eps != spec.kv_norm.eps:
+            raise ConfigError("the two latent norms share one eps")
+        if spec.window is not None and spec.window <= 0:
+            raise ConfigError(f"window must be positive, got {spec.window}")
+        self.spec = spec
+        self.dtype = ctx.dtype
+        self.position = build_position(spec.position, ctx)
+        if getattr(self.position, "pairing", "halves") != "halves" or self.position.rot_dim > spec.rot_dim:
+            raise ConfigError("the rotated part turns in pairs (i, i + n/2) of its first n numbers, n at most its size")
+        self.graph_safe = getattr(self.position, "graph_safe", True)
+        self.prompt_graph_safe = self.graph_safe and getattr(self.position, "prompt_graph_safe", False)
+        self.qk_dim = spec.head_dim + spec.rot_dim             # a head's query as the projection gives it
+        self.row = spec.kv_rank + spec.rot_dim                 # a cache row, and a head's query as the attention takes it
+        self.o_dim = spec.n_heads * spec.v_head_dim
+        # columns of the first projection: query latent, key/value latent, rotated key part, gate
+        self.first_cols = spec.q_rank + self.row + (self.o_dim if spec.gate else 0)
+        self.w_first: Optional[torch.Tensor] = None
+        self.w_uq: Optional[torch.Tensor] = None
+        self.w_uk_t: Optional[torch.Tensor] = None
+        self.w_uv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+        self.q_gain: Optional[torch.Tensor] = None
+        self.kv_gain: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        s = self.spec
+        specs = {"dq.weight": ParamSpec((s.q_rank, s.hidden)),
+                 "dq_norm.weight": ParamSpec((s.q_rank,), role="gain", init="gain"),
+                 "uq.weight": ParamSpec((s.n_heads * self.qk_dim, s.q_rank)),
+                 "dkv.weight": ParamSpec((self.row, s.hidden)),
+                 "dkv_norm.weight": ParamSpec((s.kv_rank,), role="gain", init="gain"),
+                 "uk.weight": ParamSpec((s.n_heads * s.head_dim, s.kv_rank)),
+                 "uv.weight": ParamSpec((self.o_dim, s.kv_rank)),
+                 "o_proj.weight": ParamSpec((s.hidden, self.o_dim))}
+        if s.gate:
+            specs["g.weight"] = ParamSpec((self.o_dim, s.hidden))
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        s = self.spec
+        first = [tensors["dq.weight"], tensors["dkv.weight"]] + ([tensors["g.weight"]] if s.gate else [])
+        self.w_first = torch.cat(first, dim=0).contiguous()
+        self.w_uq = tensors["uq.weight"]
+        # per head [kv_rank, head_dim]: the transposed key expansion, applied to the queries
+        self.w_uk_t = tensors["uk.weight"].view(s.n_heads, s.head_dim, s.kv_rank).transpose(1, 2).contiguous()
+        self.w_uv = tensors["uv.weight"].view(s.n_heads, s.v_head_dim, s.kv_rank).contiguous()
+        self.w_o = tensors["o_proj.weight"]
+        self.q_gain = tensors["dq_norm.weight"]
+        self.kv_gain = tensors["dkv_norm.weight"]
+
+    def flops(self, new_counts, starts) -> int:
+        s = self.spec
+        keys = 0
+        for n, s0 in zip(new_counts, starts):
+            if s.window is None:
+                keys += n * s0 + n * (n + 1) // 2
+            else:
+                keys += sum(min(s0 + i + 1, s.window) for i in range(n))
+        return 2 * sum(new_counts) * self.matrix_elements() + 2 * s.n_heads * (self.row + s.kv_rank) * keys
+
+    def activation_bytes(self, n_tokens: int) -> int:
+        s = self.spec
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        return n_tokens * ((self.first_cols + s.n_heads * self.qk_dim) * 4
+                           + (s.q_rank + s.n_heads * (self.row + s.kv_rank) + self.o_dim) * size
+                           + self.position.rot_dim * 4)
+
+    def cache_request(self) -> LatentCacheRequest:
+        return LatentCacheRequest(self.row, self.spec.window)
+
+    def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
+        s = self.spec
+        n = step.n_tokens
+        ws = step.workspace
+        if stream(step).row_scale is not None:
+            raise ConfigError("the latent attention was handed an input without its norm's scale")
+        first = ws.get("latent.first", (n, self.first_cols), torch.float32)
+        ops.gemm(xn, self.w_first, first, workspace=ws.scratch())
+        cos, sin = self.position.tables(step)
+        dims = self.position.rot_dim
+        cq = ws.get("latent.cq", (n, s.q_rank), self.dtype)
+        ops.latent_prepare(first, s.q_rank, s.kv_rank, s.rot_dim, dims, self.q_gain, self.kv_gain, s.q_norm.eps,
+                           cos, sin, cq, cache.k, cache.block_table, step.token_seq, step.token_pos,
+                           write_cache=owns_cache)
+        q = ws.get("latent.q", (n, s.n_heads * self.qk_dim), torch.float32)
+        ops.gemm(cq, self.w_uq, q, workspace=ws.scratch())
+        # the queries as the attention takes them: per head [W_uk^T q^n, rotated q^r]
+        qa = ws.get("latent.qa", (n, s.n_heads * self.row), self.dtype)
+        ops.gemm_batched(q, self.qk_dim, self.w_uk_t, qa, self.row)
+        ops.rope_heads(q, s.n_heads, self.qk_dim, s.head_dim, s.rot_dim, dims, cos, sin, qa, self.row, s.kv_rank)
+        ol = ws.get("latent.ol", (n, s.n_heads * s.kv_rank), self.dtype)
+        ops.attention(qa, ol, cache.k.unsqueeze(1), None, cache.block_table, step.token_seq, step.token_pos,
+                      s.n_heads, 1, self.row, s.scale, s.window, workspace=ws.scratch(),
+                      cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
+                      max_len=step.max_len, v_head_dim=s.kv_rank, values_in_keys=True)
+        o = ws.get("latent.o", (n, self.o_dim), self.dtype)
+        ops.gemm_batched(ol, s.kv_rank, self.w_uv, o, s.v_head_dim)
+        if s.gate:
+            ops.sigmoid_gate(o, first[:, s.q_rank + self.row:])
+        stream(step).add_product(o, self.w_o, x_accum)
+
+
+register_mixer("latent_attention", LatentAttention)

@@ -1,7 +1,8 @@
 """Dense gated feed-forward: ``y = down(act(gate(x)) * up(x))`` with no bias
 (rocml/src/forward/ffn.rs:36-107, rocml-kernels/kernels/silu_mul.hip:12-20).  Gate and up
 are one product over the concatenated weight; the residual sum is the down product's
-epilogue."""
+epilogue.  ``act`` is the spec's: ``silu`` and ``relu`` are epilogues of the gate/up product,
+``gelu_tanh`` runs as a kernel of its own behind it."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -21,8 +22,10 @@ class GatedMlp(FeedForward):
     prompt_graph_safe = True
 
     def __init__(self, spec: GatedMlpSpec, ctx: BuildContext):
-        if spec.activation != "silu":
-            raise ConfigError(f"activation {spec.activation!r} is not supported (silu only)")
+        if spec.activation not in ops.GATE_ACTIVATIONS:
+            raise ConfigError(f"activation {spec.activation!r} is not supported; known: {sorted(ops.GATE_ACTIVATIONS)}")
+        # the product's epilogue for this activation, if it has one
+        self.epilogue = {"silu": "swiglu", "relu": "relu_glu"}.get(spec.activation)
         self.spec = spec
         self.dtype = ctx.dtype
         self.w_gate_up: Optional[torch.Tensor] = None
@@ -40,12 +43,12 @@ class GatedMlp(FeedForward):
         gate, up = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         self.w_gate_up = torch.stack([gate, up], dim=1).reshape(2 * gate.shape[0], gate.shape[1]).contiguous()
         self.w_down = tensors["down_proj.weight"]
-        self.fused = self.dtype == torch.bfloat16 and self.spec.hidden % 8 == 0
+        self.fused = self.epilogue is not None and self.dtype == torch.bfloat16 and self.spec.hidden % 8 == 0
 
     def activation_bytes(self, n_tokens: int) -> int:
         s = self.spec
         size = 2 if self.dtype == torch.bfloat16 else 4
-        fused = self.dtype == torch.bfloat16 and s.hidden % 8 == 0
+        fused = self.epilogue is not None and self.dtype == torch.bfloat16 and s.hidden % 8 == 0
         return n_tokens * s.intermediate * (size + (0 if fused else 8))
 
     def takes_row_scale(self, step) -> bool:
@@ -58,13 +61,13 @@ class GatedMlp(FeedForward):
         ws = step.workspace
         h = ws.get("mlp.h", (n, s.intermediate), self.dtype)
         if self.fused:
-            ops.gemm(xn, self.w_gate_up, h, workspace=ws.scratch(), epilogue="swiglu", row_scale=stream(step).row_scale)
+            ops.gemm(xn, self.w_gate_up, h, workspace=ws.scratch(), epilogue=self.epilogue, row_scale=stream(step).row_scale)
         else:
             if stream(step).row_scale is not None:
                 raise ConfigError("the feed-forward was handed an input without its norm's scale in a step it cannot scale")
             gate_up = ws.get("mlp.gate_up", (n, 2 * s.intermediate), torch.float32)
             ops.gemm(xn, self.w_gate_up, gate_up, workspace=ws.scratch())
-            ops.swiglu(gate_up, h, interleaved=True)
+            ops.swiglu(gate_up, h, interleaved=True, activation=s.activation)
         stream(step).add_product(h, self.w_down, x_accum)
 
 

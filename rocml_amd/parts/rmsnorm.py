@@ -1,6 +1,7 @@
 """Root-mean-square norm: ``y = x / sqrt(mean(x^2) + eps) * gain`` in 32-bit
 (rocml-kernels/kernels/rmsnorm.hip:18-42); reads the 32-bit residual stream and writes
-the activation type."""
+the activation type.  With ``unit_offset`` the checkpoint stores ``gain - 1``: one is added in
+32-bit when the weight is bound, and the kernels see the gain."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -19,13 +20,14 @@ class RMSNorm(Norm):
     def __init__(self, spec: NormSpec, ctx: BuildContext):
         self.size = spec.size
         self.eps = float(spec.eps)
+        self.unit_offset = bool(getattr(spec, "unit_offset", False))
         self.gain: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.size,), role="gain", init="gain")}
+        return {"weight": ParamSpec((self.size,), role="gain", init="offset" if self.unit_offset else "gain")}
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.gain = tensors["weight"]
+        self.gain = tensors["weight"] + 1.0 if self.unit_offset else tensors["weight"]
 
     fuses_pending = True      # forward() can add a deferred product's partial sums to x itself
 

@@ -42,13 +42,13 @@ def _shard_files(path: str) -> List[str]:
 
 
 def check_tensors(expected: Dict[str, ParamSpec], names: Dict[str, str],
-                  found: Dict[str, tuple]) -> None:
+                  found: Dict[str, tuple], unused=()) -> None:
     """``found`` maps checkpoint names to ``(shape, file dtype)``.  Raises one
     ``WeightsError`` listing everything that does not fit."""
     problems: List[str] = []
     wanted = {names[k]: (k, spec) for k, spec in expected.items()}
     missing = sorted(n for n in wanted if n not in found)
-    unexpected = sorted(n for n in found if n not in wanted)
+    unexpected = sorted(n for n in found if n not in wanted and n not in set(unused))
     if missing:
         problems.append("missing tensors: " + ", ".join(missing))
     if unexpected:
@@ -86,7 +86,7 @@ def load_model(path: str, dtype="bfloat16", device="cuda") -> DecoderModel:
                 sl = f.get_slice(name)
                 found[name] = (tuple(sl.get_shape()), sl.get_dtype())
                 where[name] = file
-    check_tensors(expected, names, found)
+    check_tensors(expected, names, found, unused=arch.unused_tensors(spec))
     tensors: Dict[str, torch.Tensor] = {}
     by_file: Dict[str, List[str]] = {}
     for internal in expected:

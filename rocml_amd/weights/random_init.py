@@ -92,6 +92,8 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, dtype: torch.dtype, nor
         t = torch.ones(spec.shape, dtype=torch.float32, device=device)
         if norm_jitter:
             t += normal()
+    elif spec.init == "offset":          # a gain stored as its distance from one
+        t = normal() if norm_jitter else torch.zeros(spec.shape, dtype=torch.float32, device=device)
     elif spec.init == "zeros":
         t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
     else:
