@@ -9,7 +9,6 @@ stored ``[out, in]``.
 """
 from __future__ import annotations
 
-import math
 from typing import Dict, List, Optional
 
 import torch
@@ -31,10 +30,12 @@ def norm_one_plus(x, w, eps):
     return rms(x, eps) * (1.0 + w)
 
 
-def rotate_halves(x: torch.Tensor, positions: torch.Tensor, base: float) -> torch.Tensor:
-    """Rotates the pairs ``(i, i + n/2)`` of the last axis (width ``n``) of ``x [T, ..., n]`` by
-    ``p * base^(-2i/n)``."""
-    n = x.shape[-1]
+def rotate_halves(x: torch.Tensor, positions: torch.Tensor, base: float, dims: Optional[int] = None) -> torch.Tensor:
+    """Rotates the pairs ``(i, i + n/2)`` of the first ``n = dims`` numbers of the last axis of
+    ``x [T, ..., width]`` by ``p * base^(-2i/n)``; the rest passes unchanged."""
+    n = x.shape[-1] if dims is None else dims
+    if n < x.shape[-1]:
+        return torch.cat([rotate_halves(x[..., :n], positions, base), x[..., n:]], dim=-1)
     half = n // 2
     freq = torch.tensor([base ** (-2.0 * i / n) for i in range(half)], dtype=torch.float64)
     ang = positions.to(torch.float64)[:, None] * freq[None, :]
@@ -80,10 +81,10 @@ def latent_attention(h: torch.Tensor, t: Dict[str, torch.Tensor], pre: str, m: D
     pos = torch.arange(T)
     cq = norm_plain(h @ t[pre + "dq"].T, t[pre + "dq.norm"], eps)
     q = (cq @ t[pre + "uq"].T).view(T, H, d + r)
-    q_nope, q_rot = q[..., :d], rotate_halves(q[..., d:], pos, m["rot"]["base"])
+    q_nope, q_rot = q[..., :d], rotate_halves(q[..., d:], pos, m["rot"]["base"], m["rot"]["dims"])
     dkv = h @ t[pre + "dkv"].T
     c = norm_plain(dkv[:, :kr], t[pre + "dkv.norm"], eps)
-    k_rot = rotate_halves(dkv[:, kr:], pos, m["rot"]["base"])          # [T, r], one for all heads
+    k_rot = rotate_halves(dkv[:, kr:], pos, m["rot"]["base"], m["rot"]["dims"])          # [T, r], one for all heads
     k_nope = (c @ t[pre + "uk"].T).view(T, H, d)
     v = (c @ t[pre + "uv"].T).view(T, H, dv)
     scores = (torch.einsum("ihd,jhd->hij", q_nope, k_nope) + torch.einsum("ihd,jd->hij", q_rot, k_rot)) * m["scale"]
@@ -156,3 +157,15 @@ def forward(cfg: Dict, tensors: Dict[str, torch.Tensor], tokens, return_layers: 
     if return_layers:
         return logits, torch.stack(seen)
     return logits
+
+
+def greedy(cfg: Dict, tensors: Dict[str, torch.Tensor], prompt, n_new: int, stop=()) -> List[int]:
+    """Greedy continuation, every step a whole forward pass; a stop token ends it and is not kept."""
+    tokens, out = list(prompt), []
+    for _ in range(n_new):
+        nxt = int(torch.argmax(forward(cfg, tensors, tokens)[-1]))
+        if nxt in stop:
+            break
+        out.append(nxt)
+        tokens.append(nxt)
+    return out

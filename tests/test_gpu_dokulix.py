@@ -1,0 +1,202 @@
+"""The Dokulix decoder in the engine against the plain implementation: whole requests, tails fed
+one by one (long enough for windows and blocks to pass over decoded tokens), portions of prompts
+down to two tokens, batches of unequal requests against each alone, slots and pages used again,
+greedy generation through the Python entry point and the replay program."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import dokulix_models as dm
+from tests import helpers
+from tests.plain import dokulix_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+# the worst position's largest difference over that position's largest logit
+TOL = {"float32": 1e-4, "bfloat16": 6e-2}
+LENGTHS = {"P": [1, 2, 21, 66, 150, 211], "Q": [3, 64, 65, 131, 262], "R": [1, 8, 30, 77]}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = tmp_path_factory.mktemp("dokulix")
+    out = {}
+    for name, (cfg, seed) in dm.CONFIGS.items():
+        tensors = dm.random_tensors(cfg, seed)
+        out[name] = (dm.write_model(str(root / name), cfg, tensors), cfg, tensors)
+    return out
+
+
+def _engine(path, dtype, **kw):
+    from rocml_amd.engine import Engine
+    from rocml_amd.weights import load_model
+    kw.setdefault("max_tokens", 4096)
+    return Engine(load_model(path, dtype=dtype, device="cuda:0"), **kw)
+
+
+def _prompts(name, cfg):
+    return [helpers.random_tokens(n, cfg["vocab"], 300 + i) for i, n in enumerate(LENGTHS[name])]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q", "R"])
+def test_whole_tail_and_batches(models, name, dtype):
+    path, cfg, tensors = models[name]
+    engine = _engine(path, dtype)
+    prompts = _prompts(name, cfg)
+    refs = [plain.forward(cfg, tensors, p) for p in prompts]
+    tol = TOL[dtype]
+    for i, p in enumerate(prompts):
+        assert helpers.per_position(helpers.run_whole(engine, p), refs[i]) < tol, f"whole, length {len(p)}"
+    for i, p in enumerate(prompts):
+        # the last 100 tokens one by one: every window and block of these models passes over decoded tokens
+        assert helpers.per_position(helpers.run_tail_by_one(engine, p, 100), refs[i]) < tol, f"tail, length {len(p)}"
+    # batches of unequal requests, twice, so that slots and pages are used again; the second time in another order
+    for order in (list(range(len(prompts))), list(reversed(range(len(prompts))))):
+        batch = [prompts[i] for i in order]
+        n_prefill = [max(1, len(p) - 9 - 3 * j) for j, p in enumerate(batch)]
+        got = helpers.run_batch(engine, batch, n_prefill)
+        for j, i in enumerate(order):
+            assert helpers.per_position(got[j], refs[i]) < tol, f"batch, request of length {len(prompts[i])}"
+    engine.cache.check()
+    assert not engine.cache.lengths
+
+
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_batched_logits_equal_those_of_each_request_alone(models, name):
+    """32-bit: what else is in the batch changes nothing beyond rounding."""
+    path, cfg, tensors = models[name]
+    engine = _engine(path, "float32")
+    prompts = _prompts(name, cfg)
+    alone = [helpers.run_tail_by_one(engine, p, 12) for p in prompts]
+    got = helpers.run_batch(engine, prompts, [max(1, len(p) - 12) for p in prompts])
+    for a, g, p in zip(alone, got, prompts):
+        assert helpers.per_position(g, a) < 2e-5, f"length {len(p)}"
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 6e-2)])
+@pytest.mark.parametrize("piece", [2, 7, 64])
+def test_prompts_cut_into_portions(models, piece, dtype, tol):
+    """The engine cuts a long step into pieces itself; a piece starts anywhere in a window or a
+    block and reads what earlier pieces left in the cache."""
+    path, cfg, tensors = models["P"]
+    engine = _engine(path, dtype, max_step_tokens=piece)
+    prompts = _prompts("P", cfg)[2:5]
+    refs = [plain.forward(cfg, tensors, p) for p in prompts]
+    for p, ref in zip(prompts, refs):
+        assert helpers.per_position(helpers.run_whole(engine, p), ref) < tol, f"pieces of {piece}, length {len(p)}"
+    # three unequal requests in one step that is cut across them
+    got = helpers.run_batch(engine, prompts, [len(p) for p in prompts])
+    for g, ref in zip(got, refs):
+        assert helpers.per_position(g, ref) < tol
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_portions_given_by_the_caller(models, name):
+    """Steps of several tokens on top of a cache: portions of 2, 5, 64 and 3 tokens, then the rest."""
+    from rocml_amd.engine import StepEntry
+    path, cfg, tensors = models[name]
+    engine = _engine(path, "float32")
+    p = _prompts(name, cfg)[-1]
+    ref = plain.forward(cfg, tensors, p)
+    slot = engine.new_sequence()
+    out, at = [], 0
+    for n in [2, 5, 64, 3, len(p)]:
+        part = p[at:at + n]
+        if not part:
+            break
+        out.append(engine.step([StepEntry(slot, part, list(range(len(part))))]).cpu())
+        at += len(part)
+    engine.release(slot)
+    assert helpers.per_position(torch.cat(out), ref) < 1e-4
+
+
+def test_pages_are_given_back_and_used_again(models):
+    """A cache far smaller than the tokens that pass through it: windows and blocks give their pages
+    back while a request runs, and ended requests give back the rest."""
+    path, cfg, tensors = models["P"]
+    engine = _engine(path, "float32", max_tokens=6 * 64, max_seqs=1, max_step_tokens=64)
+    prompts = [helpers.random_tokens(n, cfg["vocab"], 500 + i) for i, n in enumerate([600, 130, 65, 200])]
+    for group in engine.cache.kv_groups:
+        assert group.n_pages < 600 // 64 + 1, "a group with a window or blocks is sized for them, not for whole requests"
+    for round_ in range(2):
+        for p in prompts:
+            ref = plain.forward(cfg, tensors, p)
+            assert helpers.per_position(helpers.run_tail_by_one(engine, p, 40), ref) < 1e-4
+            engine.cache.check()
+    assert all(g.n_free_pages == g.n_pages for g in engine.cache.kv_groups)
+
+
+@pytest.mark.parametrize("name", ["P", "R"])
+def test_greedy_generation_through_the_entry_point(models, name):
+    from rocml_amd.api import Model
+    path, cfg, tensors = models[name]
+    model = Model.load(path, dtype="float32", ctx=256, max_batch=3)
+    lengths = [5, 1, 30, 2, 70, 9, 24]
+    prompts = [helpers.random_tokens(n, cfg["vocab"], 700 + i) for i, n in enumerate(lengths)]
+    want = [plain.greedy(cfg, tensors, p, 10) for p in prompts]
+    got = model.generate(prompts, max_new_tokens=10)          # seven requests in three slots
+    assert [r.tokens for r in got] == want
+    assert model.last_stats.batches == 3
+    model.engine.cache.check()
+    assert not model.engine.cache.lengths
+    # in bfloat16 the same entry point runs; its tokens may differ from the 32-bit ones only where two logits nearly tie
+    model16 = Model.load(path, dtype="bfloat16", ctx=256, max_batch=3)
+    got16 = model16.generate(prompts, max_new_tokens=10)
+    for r, w, p in zip(got16, want, prompts):
+        for k, (a, b) in enumerate(zip(r.tokens, w)):
+            if a != b:
+                logits = plain.forward(cfg, tensors, list(p) + list(w[:k]))[-1]
+                top = torch.topk(logits, 2).values
+                assert float((top[0] - top[1]).abs()) < 0.1 * float(logits.abs().max()), "a flip away from a near tie"
+                break
+
+
+def test_long_decoding(models):
+    """300 tokens decoded one by one after a prompt of three."""
+    path, cfg, tensors = models["Q"]
+    p = helpers.random_tokens(303, cfg["vocab"], 900)
+    ref = plain.forward(cfg, tensors, p)
+    for dtype in ("float32", "bfloat16"):
+        engine = _engine(path, dtype)
+        assert helpers.per_position(helpers.run_tail_by_one(engine, p, 300), ref) < TOL[dtype]
+
+
+def test_replay_program(models, tmp_path):
+    path, cfg, tensors = models["P"]
+    vocab = cfg["vocab"]
+    prompts = {"a": helpers.random_tokens(90, vocab, 41), "b": helpers.random_tokens(7, vocab, 42)}
+    refs = {k: plain.forward(cfg, tensors, p) for k, p in prompts.items()}
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": prompts["a"][:80], "want": [0, 79]},
+                                     {"id": "b", "tokens": prompts["b"][:5], "want": [4]}], "end": []}]
+    expect = [[("a", 0), ("a", 79), ("b", 4)]]
+    for k in range(10):
+        entries = [{"id": "a", "tokens": [prompts["a"][80 + k]], "want": [0]}]
+        rows = [("a", 80 + k)]
+        if k < 2:
+            entries.append({"id": "b", "tokens": [prompts["b"][5 + k]], "want": [0]})
+            rows.append(("b", 5 + k))
+        steps.append({"step": k + 1, "entries": entries, "end": (["b"] if k == 1 else []) + (["a"] if k == 9 else [])})
+        expect.append(rows)
+    for dtype, tol in (("float32", 1e-4), ("bfloat16", 6e-2)):
+        out_dir = str(tmp_path / dtype)
+        cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", path, "--dtype", dtype,
+               "--out", out_dir, "--max-tokens", "128"]
+        proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+        for step in steps:
+            proc.stdin.write(json.dumps(step) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == f"done {step['step']}"
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+        for step, rows in zip(steps, expect):
+            got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{step['step']}.f32"), dtype="<f4").reshape(-1, vocab))
+            want = torch.stack([refs[r][i] for r, i in rows])
+            assert helpers.per_position(got, want) < tol, f"step {step['step']} in {dtype}"
