@@ -29,18 +29,34 @@ struct AttnArgs {
     int n_splits_hint;
     const DecodeProj* proj;     // decode only: the step's q/k/v projection instead of q and an appended cache
     const PrefillProj* prefill_proj = nullptr;      // prompts: the projection instead of prepared queries
+    MaskExtra extra = MaskExtra{};                  // blocks of positions, distance slopes, sink
+    bool has_extra = false;
 };
 
 template <int D, bool FUSED, int AHEAD, int WAVES>
 static int launch_decode_kernel(const AttnArgs& a, int n_splits, float* part_o, float* part_ml, hipStream_t stream) {
     int group = a.hq / a.hkv;
     int lds = WAVES * group * (D + 4) * (int)sizeof(float);
+    dim3 grid(n_splits, a.hkv, a.n_tokens);
+    if constexpr (!FUSED) {
+        if (a.has_extra) {
+            static int allowed_extra = 0;
+            if (lds > allowed_extra) {
+                if (allow_lds(attn_decode_mfma_kernel<D, false, AHEAD, WAVES, true>, lds)) return 1;
+                allowed_extra = lds;
+            }
+            attn_decode_mfma_kernel<D, false, AHEAD, WAVES, true><<<grid, 64 * WAVES, lds, stream>>>(
+                a.q, a.out, const_cast<bf16_t*>(a.kcache), const_cast<bf16_t*>(a.vcache), a.block_table, a.bt_width,
+                a.token_seq, a.token_pos, a.hq, a.hkv, a.scale * LOG2E, a.window, n_splits, part_o, part_ml,
+                DecodeProj{}, a.extra);
+            return 0;
+        }
+    }
     static int allowed = 0;
     if (lds > allowed) {
         if (allow_lds(attn_decode_mfma_kernel<D, FUSED, AHEAD, WAVES>, lds)) return 1;
         allowed = lds;
     }
-    dim3 grid(n_splits, a.hkv, a.n_tokens);
     attn_decode_mfma_kernel<D, FUSED, AHEAD, WAVES><<<grid, 64 * WAVES, lds, stream>>>(
         a.q, a.out, const_cast<bf16_t*>(a.kcache), const_cast<bf16_t*>(a.vcache), a.block_table, a.bt_width,
         a.token_seq, a.token_pos, a.hq, a.hkv, a.scale * LOG2E, a.window, n_splits, part_o, part_ml,
@@ -102,10 +118,15 @@ static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
     if (!ready) {
         if (allow_lds(attn_prefill_mfma_kernel<D, false>, PrefillLds<D>::BYTES)) return 1;
         if (allow_lds(attn_prefill_mfma_kernel<D, true>, PrefillLds<D>::BYTES)) return 1;
+        if (allow_lds(attn_prefill_mfma_kernel<D, false, true>, PrefillLds<D>::BYTES)) return 1;
         ready = true;
     }
     dim3 grid(a.total_q_tiles * a.hq);
-    if (a.prefill_proj)
+    if (a.has_extra)
+        attn_prefill_mfma_kernel<D, false, true><<<grid, AM_THREADS, PrefillLds<D>::BYTES, stream>>>(
+            a.q, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos,
+            a.hq, a.hkv, a.scale * LOG2E, a.window, PrefillProj{}, a.extra);
+    else if (a.prefill_proj)
         attn_prefill_mfma_kernel<D, true><<<grid, AM_THREADS, PrefillLds<D>::BYTES, stream>>>(
             nullptr, a.out, a.kcache, a.vcache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos,
             a.hq, a.hkv, a.scale * LOG2E, a.window, *a.prefill_proj);
@@ -146,7 +167,8 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     ROCML_REQUIRE(v_in_k || vcache, "attention: no value cache");
     ROCML_REQUIRE(dv <= AG_BLOCK * AG_MAX_D_PER_THREAD, "attention: value head size %d exceeds %d", dv,
                   AG_BLOCK * AG_MAX_D_PER_THREAD);
-    bool plain_features = dv == d && !v_in_k && chunk == 0 && !slopes && !sink;
+    bool plain_features = dv == d && !v_in_k;          // what the matrix-core kernels need
+    bool has_extra = chunk > 0 || slopes || sink;
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0 && page_size > 0 && bt_width > 0,
                   "attention: bad sizes T=%d Hq=%d Hkv=%d D=%d page=%d width=%d", n_tokens, hq, hkv,
                   d, page_size, bt_width);
@@ -177,6 +199,8 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
         AttnArgs a{(const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,
                    bt_width, token_seq, token_pos, cu_seqlens, n_seqs, n_tokens, (int)total_q_tiles, max_len, hq, hkv,
                    scale, window, workspace, workspace_bytes, n_splits, nullptr};
+        a.extra = MaskExtra{chunk, slopes, sink};
+        a.has_extra = has_extra;
         int rc = decode ? BY_HEAD_DIM(launch_decode_plain, d, a, stream) : BY_HEAD_DIM(launch_prefill, d, a, stream);
         if (rc) return rc;
         ROCML_CHECK_LAUNCH("attention");

@@ -65,14 +65,25 @@ struct DecodeProj {
 // keys end before it.  A page belongs to one split, so no other block reads that row.
 // WAVES: 4, or 8 for launches of at most one block a CU whose blocks have many pieces: a wave
 // then has half as many, and the pieces of a block travel in half as many trips.
-template <int D, bool FUSED, int AHEAD, int WAVES>
+// EXTRA: the layer's mask and scores have more to them than a window (MaskExtra): blocks of
+// positions, a penalty on distance, a sink.  A kernel without EXTRA is the same code as before.
+struct MaskExtra {
+    int chunk;              // > 0: a query sees the keys of its own block of `chunk` positions (counted from 0) up to itself
+    const float* slopes;    // [Hq] or null: slope * (query position - key position) is taken off a score
+    int sink;               // one more term exp(0) in the softmax's denominator, with no value
+};
+constexpr float AM_LOG2E = 1.4426950408889634f;
+
+template <int D, bool FUSED, int AHEAD, int WAVES, bool EXTRA = false>
 __global__ void __launch_bounds__(64 * WAVES)
 attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                         bf16_t* kcache, bf16_t* vcache,
                         const int* __restrict__ block_table, int bt_width,
                         const int* __restrict__ token_seq, const int* __restrict__ token_pos, int hq,
                         int hkv, float scale_log2e, int window, int n_splits,
-                        float* __restrict__ part_o, float* __restrict__ part_ml, DecodeProj pj) {
+                        float* __restrict__ part_o, float* __restrict__ part_ml, DecodeProj pj,
+                        MaskExtra mx = MaskExtra{}) {
+    static_assert(!(FUSED && EXTRA), "the kernel that reads the projection knows plain layers only");
     constexpr int KD = D / 32;      // MFMA steps along D for the scores
     constexpr int DT = D / 16;      // 16-row tiles of the output
     constexpr int THREADS = 64 * WAVES;
@@ -91,6 +102,15 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     for (int i = 0; i < 4; ++i) early[i] = pages[split + i * n_splits < bt_width ? split + i * n_splits : 0];
     int len = token_pos[t] + 1;
     int lo = window > 0 ? max(0, len - window) : 0;
+    bool from_start = window == 0;                  // the sequence's first pages are the split's first pages
+    float slope_l2 = 0.f;
+    if constexpr (EXTRA) {
+        if (mx.chunk > 0) {
+            lo = (len - 1) - (len - 1) % mx.chunk;
+            from_start = false;
+        }
+        if (mx.slopes) slope_l2 = mx.slopes[kvh * group + min(col, group - 1)] * AM_LOG2E;
+    }
     int first_page = lo / AM_PAGE;
     int n_pages = (len + AM_PAGE - 1) / AM_PAGE - first_page;
     // split s takes pages s, s + n_splits, ...: the splits of a sequence, which run side by side,
@@ -111,7 +131,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         // (the page index is the same for all lanes: a scalar load)
         int round = __builtin_amdgcn_readfirstlane(piece >> 1), half = piece & 1;
         int phys;
-        if (window == 0 && round < 4)
+        if (from_start && round < 4)
             phys = round == 0 ? early[0] : round == 1 ? early[1] : round == 2 ? early[2] : early[3];
         else
             phys = pages[first_page + split + round * n_splits];
@@ -252,6 +272,10 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         vnew_lds = sm_vnew;
     }
     float m = -INFINITY, l = 0.f;
+    if constexpr (EXTRA) {
+        // the sink is one key of score 0 and value 0: it enters once, in the first wave of the first split
+        if (mx.sink && split == 0 && wave == 0) { m = 0.f; l = 1.f; }
+    }
     f32x4_t o[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -278,6 +302,7 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             for (int i = 0; i < 4; ++i) {
                 int key = key0 + g * 8 + u * 4 + i;
                 float v = (key >= from && key < to) ? s[u][i] * scale_log2e : -INFINITY;
+                if constexpr (EXTRA) v -= slope_l2 * (float)(len - 1 - key);
                 s[u][i] = v;
                 mx = fmaxf(mx, v);
             }
@@ -441,15 +466,22 @@ struct PrefillProj {
     const float* cos_t; const float* sin_t;             // [T, D/2], null: no rotation
 };
 
-template <int D, bool QPREP>
+__device__ __forceinline__ int am_first_key(int pos, int window, int chunk) {
+    if (chunk > 0) return pos - pos % chunk;
+    return window > 0 ? max(0, pos - window + 1) : 0;
+}
+
+template <int D, bool QPREP, bool EXTRA = false>
 __global__ void __launch_bounds__(AM_THREADS, D <= 128 ? 2 : 1)
 attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                          const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                          const int* __restrict__ block_table, int bt_width,
                          const int* __restrict__ cu_seqlens, int n_seqs,
                          const int* __restrict__ token_pos, int hq, int hkv, float scale_log2e,
-                         int window, PrefillProj pj) {
+                         int window, PrefillProj pj, MaskExtra mx = MaskExtra{}) {
+    static_assert(!(QPREP && EXTRA), "the kernel that prepares its queries knows plain layers only");
     using L = PrefillLds<D>;
+    const int chunk = EXTRA ? mx.chunk : 0;
     constexpr int KK = D / 16;      // MFMA steps along D for the scores
     constexpr int DT = D / 32;      // 32-row tiles of the output
     extern __shared__ uint4 am_smem[];
@@ -485,10 +517,16 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     int my_row = w_lo + col;
     bool row_ok = my_row < n_new;
     int my_pos = pos0 + my_row;
-    int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
-    int blk_first_key = window > 0 ? max(0, pos0 + row_lo - window + 1) : 0;
+    // (the first key a position sees does not decrease with the position, for windows and for blocks)
+    int my_lo = am_first_key(my_pos, window, chunk);
+    int blk_first_key = am_first_key(pos0 + row_lo, window, chunk);
     int blk_last_key = pos0 + row_hi;
-    int wave_first_key = window > 0 ? max(0, pos0 + w_lo - window + 1) : 0;
+    int wave_first_key = am_first_key(pos0 + w_lo, window, chunk);
+    // a distance penalty in the units of the raw dot products (they are scaled when exponentiated)
+    float kslope = 0.f;
+    if constexpr (EXTRA) {
+        if (mx.slopes) kslope = mx.slopes[h] * AM_LOG2E / scale_log2e;
+    }
     int wave_last_key = pos0 + w_hi;
 
     // Q^T operand: column = query row, 8 values of D per lane and step.
@@ -554,6 +592,9 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
         }
     }
     float m = -INFINITY, l = 0.f;
+    if constexpr (EXTRA) {
+        if (mx.sink) { m = 0.f; l = 1.f; }            // one key of score 0 and value 0 in every row
+    }
     f32x16_t o[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i)
@@ -577,7 +618,7 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
     // the wave's rows see every key of a 32-key piece when the piece lies at or below the first
     // row's position and at or above the last row's window start; only then masking is skipped
     int wave_min_pos = pos0 + w_lo;
-    int wave_max_lo = window > 0 ? max(0, pos0 + w_hi - window + 1) : 0;
+    int wave_max_lo = am_first_key(pos0 + w_hi, window, chunk);
     bool wave_full = w_hi - w_lo == 31;
     AM_LOAD_PAGE(first_page)
     for (int lpage = first_page; lpage <= last_page; ++lpage) {
@@ -635,6 +676,15 @@ attn_prefill_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                 for (int e = 0; e < 16; ++e) {
                     int key = key0 + 8 * (e >> 2) + 4 * h2 + (e & 3);
                     s[e] = (row_ok && key <= my_pos && key >= my_lo) ? s[e] : -INFINITY;
+                }
+            }
+            if constexpr (EXTRA) {
+                if (kslope != 0.f) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        int key = key0 + 8 * (e >> 2) + 4 * h2 + (e & 3);
+                        s[e] -= kslope * (float)(my_pos - key);
+                    }
                 }
             }
             float mx = s[0];

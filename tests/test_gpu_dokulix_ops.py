@@ -271,3 +271,48 @@ def test_norm_whose_weight_is_stored_around_zero():
         out = torch.empty((9, 40), dtype=torch.float32, device=DEV)
         norm.forward(x.to(DEV), out)
         assert float((out.cpu() - ref).abs().max()) < 1e-5
+
+
+def _run_fast_attention(q, k, v, scale, first, window=None, chunk=None, slopes=None, sink=False, decode=False, n_splits=0):
+    """The matrix-core kernels (bfloat16): the queries at positions ``first ..`` of one sequence as one
+    prompt step, or, with ``decode``, each as the one new token of a sequence of its own."""
+    from rocml_amd import ops
+    T, H, D = q.shape
+    G = k.shape[1]
+    n_pages = (T + PAGE - 1) // PAGE + 2
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(T + first))
+    kc = _paged(k, n_pages, perm, False).to(torch.bfloat16).to(DEV)
+    vc = _paged(v, n_pages, perm, True).to(torch.bfloat16).to(DEV)
+    n = T - first
+    rows = n if decode else 1
+    table = torch.full((rows, 8), -1, dtype=torch.int32)
+    table[:, :(T + PAGE - 1) // PAGE] = perm[:(T + PAGE - 1) // PAGE].to(torch.int32)
+    qs = q[first:].reshape(n, H * D).to(torch.bfloat16).to(DEV).contiguous()
+    out = torch.empty((n, H * D), dtype=torch.bfloat16, device=DEV)
+    seq = (torch.arange(n) if decode else torch.zeros(n)).to(torch.int32).to(DEV)
+    pos = torch.arange(first, T, dtype=torch.int32, device=DEV)
+    cu = (torch.arange(n + 1) if decode else torch.tensor([0, n])).to(torch.int32).to(DEV)
+    ws = torch.empty(1 << 24, dtype=torch.uint8, device=DEV)
+    ops.attention(qs, out, kc, vc, table.to(DEV), seq, pos, H, G, D, scale, window, algo=ops.ATTN_MFMA, workspace=ws,
+                  cu_seqlens=cu, max_new=1 if decode else n, q_counts=[1] * n if decode else [n], max_len=T,
+                  n_splits=n_splits, chunk=chunk, slopes=None if slopes is None else slopes.to(DEV), sink=sink)
+    return out.float().cpu().view(n, H, D)
+
+
+@pytest.mark.parametrize("H,G,D,chunk", [(8, 2, 64, 100), (6, 1, 96, 130), (4, 4, 128, 64), (2, 2, 32, 7)])
+@pytest.mark.parametrize("decode", [False, True])
+def test_matrix_core_kernels_take_blocks_slopes_and_sink(H, G, D, chunk, decode):
+    gen = torch.Generator().manual_seed(H * D + chunk)
+    T = 333
+    q, k, v = (torch.randn(T, n, D, generator=gen).to(torch.bfloat16).float() for n in (H, G, G))
+    slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)])
+    scale = D ** -0.5
+    for first, sl, sink, splits in ((0, slopes, True, 0), (150, None, True, 3), (40, slopes, False, 1)):
+        ref = _attend(q, k, v, scale, plain.chunk_mask(T, chunk), sl, sink)[first:]
+        got = _run_fast_attention(q, k, v, scale, first, chunk=chunk, slopes=sl, sink=sink, decode=decode, n_splits=splits)
+        err = (got - ref).abs().amax(dim=(1, 2))
+        assert float(err.max()) < 2e-2 * max(1.0, float(ref.abs().max())), f"position {first + int(err.argmax())}"
+    # and what they did before: a window, no extras
+    ref = _attend(q, k, v, scale, plain.window_mask(T, 70), None, False)[20:]
+    got = _run_fast_attention(q, k, v, scale, 20, window=70, decode=decode)
+    assert float((got - ref).abs().max()) < 2e-2 * max(1.0, float(ref.abs().max()))
