@@ -6,6 +6,7 @@
 #include "common.h"
 #include "attention_generic.h"
 #include "attention_mfma.h"
+#include "attention_latent.h"
 
 ROCML_LAST_ERROR_FN(attention)
 
@@ -137,6 +138,42 @@ static int launch_prefill(const AttnArgs& a, hipStream_t stream) {
     return 0;
 }
 
+// Attention over latent rows (attention_latent.h): a block per 64 rows of work and key split.
+struct LatentArgs {
+    const bf16_t* q; bf16_t* out; const bf16_t* cache; const int* block_table; int bt_width;
+    const int* cu_seqlens; int n_seqs; const int* token_pos; int n_tokens; int n_heads; int dk; int dv;
+    float scale; int window; int tiles; void* workspace; long long workspace_bytes;
+};
+
+template <int KD, int DT>
+static int launch_latent(const LatentArgs& a, hipStream_t stream) {
+    using L = LatentLds<KD, DT>;
+    static bool ready = false;
+    if (!ready) {
+        if (allow_lds(attn_latent_mfma_kernel<KD, DT>, L::BYTES)) return 1;
+        ready = true;
+    }
+    // Splits of the key range: enough blocks for two a CU, at most one per piece the rows can see.
+    // The choice follows the launch's shape (rows, window, width of the block table), not the lengths.
+    int cus = cu_count();
+    int pieces = a.window > 0 ? a.window / AL_KEYS + 2 : a.bt_width * (AM_PAGE / AL_KEYS);
+    int n_splits = 2 * cus / a.tiles;
+    if (n_splits > pieces) n_splits = pieces;
+    if (n_splits > 64) n_splits = 64;
+    long long rows = (long long)a.n_tokens * a.n_heads;
+    long long per_split = rows * (a.dv + 2) * (long long)sizeof(float);
+    if (n_splits > 1 && per_split * n_splits > a.workspace_bytes) n_splits = a.workspace ? (int)(a.workspace_bytes / per_split) : 1;
+    if (n_splits < 1) n_splits = 1;
+    float* part_o = (float*)a.workspace;
+    float* part_ml = part_o ? part_o + rows * n_splits * a.dv : nullptr;
+    attn_latent_mfma_kernel<KD, DT><<<dim3(a.tiles, n_splits), 256, L::BYTES, stream>>>(
+        a.q, a.out, a.cache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos, a.n_heads, a.dk, a.dv,
+        a.scale * LOG2E, a.window, n_splits, part_o, part_ml);
+    if (n_splits > 1)
+        attn_latent_reduce_kernel<<<(unsigned)rows, a.dv >= 256 ? 256 : 128, 0, stream>>>(part_o, part_ml, a.out, n_splits, a.dv);
+    return 0;
+}
+
 static bool mfma_head_dim(int d) { return d == 32 || d == 64 || d == 96 || d == 128 || d == 192 || d == 256; }
 
 #define BY_HEAD_DIM(fn, d, ...)                       \
@@ -191,10 +228,32 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
     ROCML_REQUIRE(total_q_tiles * hq < (1ll << 31), "attention: too many query tiles");
     bool mfma_ok = plain_features && dtype == ROCML_BF16 && page_size == AM_PAGE && mfma_head_dim(d) && max_new >= 1 &&
                    (decode ? hq / hkv <= 16 : (cu_seqlens != nullptr && n_seqs > 0 && total_q_tiles > 0));
-    if (algo == ATTN_MFMA)
+    if (algo == ATTN_MFMA && !v_in_k)
         ROCML_REQUIRE(mfma_ok, "attention: the MFMA kernels need bfloat16, pages of 64 positions, a head size "
                                "of 32, 64, 96, 128, 192 or 256, at most 16 query heads per kv head in decode and "
                                "the sequence offsets in prefill (D=%d page=%d group=%d)", d, page_size, hq / hkv);
+    // one shared key/value head whose values lie in its key rows: the kernel for latent rows
+    bool latent_ok = v_in_k && !has_extra && dtype == ROCML_BF16 && page_size == AM_PAGE && hkv == 1 && d % 8 == 0 &&
+                     dv % 8 == 0 && d <= 576 && dv <= 512 && max_new >= 1 && cu_seqlens && n_seqs > 0 && q_counts;
+    if (algo == ATTN_MFMA && v_in_k)
+        ROCML_REQUIRE(latent_ok, "attention: the matrix-core kernel for values in the key rows needs bfloat16, pages of 64, one "
+                                 "key/value head, sizes that are multiples of 8 up to 576 and 512, and the sequence offsets "
+                                 "(D=%d Dv=%d Hkv=%d)", d, dv, hkv);
+    if (latent_ok && algo != ATTN_PLAIN) {
+        long long tiles = 0;
+        for (int b = 0; b < n_seqs; ++b) tiles += ((long long)q_counts[b] * hq + AL_ROWS - 1) / AL_ROWS;
+        ROCML_REQUIRE(tiles > 0 && tiles < (1ll << 31), "attention: %lld row tiles", tiles);
+        LatentArgs a{(const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, block_table, bt_width, cu_seqlens, n_seqs,
+                     token_pos, n_tokens, hq, d, dv, scale, window, (int)tiles, workspace, workspace_bytes};
+        int kd = (d + 31) / 32, dt = (dv + 15) / 16;
+        int rc = kd <= 3 && dt <= 4     ? launch_latent<3, 4>(a, stream)
+                 : kd <= 6 && dt <= 8   ? launch_latent<6, 8>(a, stream)
+                 : kd <= 10 && dt <= 16 ? launch_latent<10, 16>(a, stream)
+                                        : launch_latent<18, 32>(a, stream);
+        if (rc) return rc;
+        ROCML_CHECK_LAUNCH("attention over latent rows");
+        return 0;
+    }
     if (mfma_ok && algo != ATTN_PLAIN) {
         AttnArgs a{(const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table,
                    bt_width, token_seq, token_pos, cu_seqlens, n_seqs, n_tokens, (int)total_q_tiles, max_len, hq, hkv,

@@ -1,0 +1,240 @@
+// bfloat16 attention over a cache of latent rows on the gfx950 matrix cores.
+//
+// The cache holds one row of DK numbers per position, [page, 64, DK]; all query heads share it (one
+// key/value "head"), a key is the whole row and its value is the row's first DV numbers.  A layer
+// whose keys and values are expanded from a latent vector reaches this form by folding the key
+// expansion into its queries and the value expansion into a product behind the attention.
+//
+// Rows of work are the (token, head) pairs of a step: the queries [T, H, DK] and the outputs
+// [T, H, DV] are plain matrices of T * H rows, and row r of a sequence's new tokens stands at
+// position pos0 + r / H.  A block takes 64 consecutive rows of one sequence (16 per wave: the 16
+// columns of an MFMA) and one split of their keys; keys come 32 at a time through LDS, once as
+// rows (the first product, S^T = K Q^T, reads 8 numbers of a key per lane) and once transposed
+// (the second, O^T = V^T P^T, reads 8 keys of a number per lane): the transposition happens on
+// the way into LDS, the cache keeps the rows only.  With many rows per sequence (a prompt) the
+// 64 rows share every key they load; with few (a decode step: H rows per sequence) the key range
+// is cut into splits whose partial results a second kernel merges by log-sum-exp, in split order.
+//
+// Online softmax per column as in attention_mfma.h; scores scaled after the dot product, base-2
+// exponentials.  A window limits the keys of a row to (pos - window, pos].
+// KD: 32-number steps of the first product (DK <= 32 KD), DT: 16-number tiles of the output
+// (DV <= 16 DT); numbers beyond DK or DV are zeros in LDS and in the query operand.
+#pragma once
+#include "attention_mfma.h"
+
+constexpr int AL_ROWS = 64;           // rows of a block
+constexpr int AL_KEYS = 32;           // keys of a piece
+constexpr int AL_VROW = AL_KEYS + 8;  // bf16 per row of the transposed piece (16 bytes of padding)
+
+template <int KD, int DT>
+struct LatentLds {
+    static constexpr int K_ROW = KD * 32 + 8;                               // bf16 per key row
+    static constexpr int BYTES = (AL_KEYS * K_ROW + DT * 16 * AL_VROW) * 2;
+};
+
+template <int KD, int DT>
+__global__ void __launch_bounds__(256)
+attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
+                        const int* __restrict__ block_table, int bt_width, const int* __restrict__ cu_seqlens,
+                        int n_seqs, const int* __restrict__ token_pos, int n_heads, int dk, int dv,
+                        float scale_log2e, int window, int n_splits, float* __restrict__ part_o,
+                        float* __restrict__ part_ml) {
+    using L = LatentLds<KD, DT>;
+    extern __shared__ uint4 al_smem[];
+    bf16_t* sk = (bf16_t*)al_smem;                    // [AL_KEYS][K_ROW]
+    bf16_t* sv = sk + AL_KEYS * L::K_ROW;             // [DT * 16][AL_VROW]
+    int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int g = lane >> 4, col = lane & 15;
+    int split = blockIdx.y;
+    // which sequence and which of its row tiles
+    int tile = blockIdx.x, b = 0, tok0 = 0, n_rows = 0;
+    for (; b < n_seqs; ++b) {
+        tok0 = cu_seqlens[b];
+        n_rows = (cu_seqlens[b + 1] - tok0) * n_heads;
+        int tiles = (n_rows + AL_ROWS - 1) / AL_ROWS;
+        if (tile < tiles) break;
+        tile -= tiles;
+    }
+    if (b >= n_seqs) return;
+    const int* pages = block_table + (size_t)b * bt_width;
+    int pos0 = token_pos[tok0];
+    int row0 = tile * AL_ROWS, row1 = min(n_rows, row0 + AL_ROWS) - 1;        // the block's rows
+    int my_row = row0 + wave * 16 + col;
+    bool row_ok = my_row <= row1;
+    int my_pos = pos0 + (row_ok ? my_row : row1) / n_heads;
+    int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+    int w_first = row0 + wave * 16, w_last = min(row1, w_first + 15);
+    bool wave_active = w_first <= row1;
+    int wave_lo = window > 0 ? max(0, pos0 + w_first / n_heads - window + 1) : 0;     // first key any of the wave's rows sees
+    int wave_hi = pos0 + w_last / n_heads;                                            // last key
+    int blk_lo = window > 0 ? max(0, pos0 + row0 / n_heads - window + 1) : 0;
+    int blk_hi = pos0 + row1 / n_heads;
+    int first_piece = blk_lo / AL_KEYS, last_piece = blk_hi / AL_KEYS;
+
+    // zeros where the sizes stop short of the tiles: they are never written again
+    for (int i = tid; i < L::BYTES / 16; i += 256) al_smem[i] = make_uint4(0u, 0u, 0u, 0u);
+
+    // Q^T operand: column = row of work, 8 numbers per lane and step
+    size_t grow = (size_t)tok0 * n_heads + (row_ok ? my_row : row1);
+    bf16x8_t qf[KD];
+    {
+        const bf16_t* qrow = q + grow * dk + g * 8;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            bool ok = row_ok && kd * 32 + g * 8 < dk;
+            uint4 v = ok ? *(const uint4*)(qrow + kd * 32) : make_uint4(0u, 0u, 0u, 0u);
+            qf[kd] = __builtin_bit_cast(bf16x8_t, v);
+        }
+    }
+    float m = -INFINITY, l = 0.f;
+    f32x4_t o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // A piece on its way: a thread takes pairs of keys (2 kp, 2 kp + 1) and 8 numbers of both, so
+    // that the transposed copy is written two keys (4 bytes) at a time.
+    int dk8 = dk / 8, dv8 = dv / 8;
+    int items = (AL_KEYS / 2) * dk8;
+    constexpr int MAX_ITEMS = (AL_KEYS / 2) * (KD * 4) / 256 + 1;
+    uint4 ra[MAX_ITEMS], rb[MAX_ITEMS];
+    auto request_piece = [&](int piece) {
+        int key0 = piece * AL_KEYS;
+        int phys = max(pages[key0 / AM_PAGE], 0);       // (a page that is not there holds no visible key)
+        const bf16_t* base = cache + ((size_t)phys * AM_PAGE + key0 % AM_PAGE) * dk;
+#pragma unroll
+        for (int i = 0; i < MAX_ITEMS; ++i) {
+            int w = tid + i * 256;
+            if (w < items) {
+                int kp = w / dk8, dc = w - kp * dk8;
+                ra[i] = *(const uint4*)(base + (size_t)(2 * kp) * dk + dc * 8);
+                rb[i] = *(const uint4*)(base + (size_t)(2 * kp + 1) * dk + dc * 8);
+            }
+        }
+    };
+    auto store_piece = [&]() {
+#pragma unroll
+        for (int i = 0; i < MAX_ITEMS; ++i) {
+            int w = tid + i * 256;
+            if (w < items) {
+                int kp = w / dk8, dc = w - kp * dk8;
+                *(uint4*)(sk + (2 * kp) * L::K_ROW + dc * 8) = ra[i];
+                *(uint4*)(sk + (2 * kp + 1) * L::K_ROW + dc * 8) = rb[i];
+                if (dc < dv8) {
+                    const uint32_t a[4] = {ra[i].x, ra[i].y, ra[i].z, ra[i].w};
+                    const uint32_t c[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+                    uint32_t* dst = (uint32_t*)(sv + (dc * 8) * AL_VROW + 2 * kp);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        // numbers 2j and 2j + 1 of both keys: (key 2kp, key 2kp + 1) side by side
+                        dst[(2 * j) * (AL_VROW / 2)] = (a[j] & 0xffffu) | (c[j] << 16);
+                        dst[(2 * j + 1) * (AL_VROW / 2)] = (a[j] >> 16) | (c[j] & 0xffff0000u);
+                    }
+                }
+            }
+        }
+    };
+
+    int piece = first_piece + split;
+    if (piece <= last_piece) request_piece(piece);
+    for (; piece <= last_piece; piece += n_splits) {
+        __syncthreads();                 // the piece before has been multiplied (first round: the zeros are written)
+        store_piece();
+        __syncthreads();
+        if (piece + n_splits <= last_piece) request_piece(piece + n_splits);
+        int key0 = piece * AL_KEYS;
+        if (!wave_active || key0 > wave_hi || key0 + AL_KEYS - 1 < wave_lo) continue;      // wave-uniform
+        // scores of 2 x 16 keys: row r of tile u is key 8 (r / 4) + 4 u + r % 4, so that element i of
+        // s[u] in lane (g, col) is key 8 g + 4 u + i of the column's row of work
+        f32x4_t s[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            const bf16_t* krow = sk + (8 * (col >> 2) + 4 * u + (col & 3)) * L::K_ROW + g * 8;
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kd * 32));
+                s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kd], s[u], 0, 0, 0);
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                int key = key0 + g * 8 + u * 4 + i;
+                float v = (row_ok && key >= my_lo && key <= my_pos) ? s[u][i] * scale_log2e : -INFINITY;
+                s[u][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float m_new = fmaxf(m, mx);
+        float m_use = m_new == -INFINITY ? 0.f : m_new;
+        float corr = fast_exp2(m - m_use);
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                s[u][i] = fast_exp2(s[u][i] - m_use);
+                sum += s[u][i];
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l = l * corr + sum;
+        m = m_new;
+        // P^T operand: slots 0..7 = keys 8g .. 8g+7
+        bf16x8_t pf = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(s[0][0], s[0][1]), pack_bf16x2(s[0][2], s[0][3]),
+                                                              pack_bf16x2(s[1][0], s[1][1]), pack_bf16x2(s[1][2], s[1][3])));
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sv + (dt * 16 + col) * AL_VROW + g * 8));
+            o[dt] = o[dt] * corr;
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
+        }
+    }
+    if (!row_ok) return;
+    // element i of o[dt] is number 16 dt + 4 g + i of the column's row
+    if (n_splits == 1) {
+        float inv = 1.0f / l;
+        bf16_t* orow = out + grow * dv;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            int d = dt * 16 + 4 * g;
+            if (d < dv)       // (dv is a multiple of 8: four numbers are inside or outside together)
+                *(uint2*)(orow + d) = make_uint2(pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv), pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv));
+        }
+    } else {
+        size_t slot = grow * n_splits + split;
+        float* po = part_o + slot * dv;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            int d = dt * 16 + 4 * g;
+            if (d < dv) *(float4*)(po + d) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
+        }
+        if (g == 0) {
+            part_ml[slot * 2] = m;
+            part_ml[slot * 2 + 1] = l;
+        }
+    }
+}
+
+// Log-sum-exp merge of the splits of a row, in split order; one block per row, a thread per number.
+__global__ void attn_latent_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                          bf16_t* __restrict__ out, int n_splits, int dv) {
+    size_t row = blockIdx.x;
+    const float* ml = part_ml + row * n_splits * 2;
+    float mm = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, ml[s * 2]);
+    float ll = 0.f;
+    for (int s = 0; s < n_splits; ++s) ll += ml[s * 2] == -INFINITY ? 0.f : ml[s * 2 + 1] * fast_exp2(ml[s * 2] - mm);
+    float inv = 1.0f / ll;
+    for (int d = threadIdx.x; d < dv; d += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            float w = ml[s * 2] == -INFINITY ? 0.f : fast_exp2(ml[s * 2] - mm);
+            acc += part_o[(row * n_splits + s) * dv + d] * w;
+        }
+        out[row * dv + d] = f32_to_bf16(acc * inv);
+    }
+}

@@ -316,3 +316,44 @@ def test_matrix_core_kernels_take_blocks_slopes_and_sink(H, G, D, chunk, decode)
     ref = _attend(q, k, v, scale, plain.window_mask(T, 70), None, False)[20:]
     got = _run_fast_attention(q, k, v, scale, 20, window=70, decode=decode)
     assert float((got - ref).abs().max()) < 2e-2 * max(1.0, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("H,DK,DV,window", [(5, 48, 40, 33), (16, 96, 64, 100), (8, 192, 128, None), (16, 576, 512, 70), (3, 320, 256, 64)])
+@pytest.mark.parametrize("decode", [False, True])
+def test_matrix_core_kernel_for_latent_rows(H, DK, DV, window, decode):
+    """Two sequences of unequal lengths whose rows of work (token, head) share one key/value head with the
+    values in the key rows; a prompt step on top of cached positions, and a decode step."""
+    from rocml_amd import ops
+    gen = torch.Generator().manual_seed(H + DK)
+    lens, firsts = (300, 131), ((0, 37) if not decode else (299, 130))
+    n_pages = 12
+    perm = torch.randperm(n_pages, generator=gen)
+    cache = torch.zeros((n_pages, PAGE, DK), dtype=torch.bfloat16)
+    table = torch.full((2, 8), -1, dtype=torch.int32)
+    qs, refs, pos, seq, at = [], [], [], [], 0
+    for b, (T, first) in enumerate(zip(lens, firsts)):
+        q = torch.randn(T, H, DK, generator=gen).to(torch.bfloat16).float()
+        k = torch.randn(T, 1, DK, generator=gen).to(torch.bfloat16).float()
+        pages = perm[at:at + (T + PAGE - 1) // PAGE]
+        at += len(pages)
+        table[b, :len(pages)] = pages.to(torch.int32)
+        for j in range(T):
+            cache[int(pages[j // PAGE]), j % PAGE] = k[j, 0].to(torch.bfloat16)
+        visible = plain.window_mask(T, window) if window else plain.window_mask(T, T)
+        refs.append(_attend(q, k, k[:, :, :DV], DK ** -0.5, visible, None, False)[first:])
+        qs.append(q[first:])
+        pos += list(range(first, T))
+        seq += [b] * (T - first)
+    n = len(pos)
+    qd = torch.cat(qs).reshape(n, H * DK).to(torch.bfloat16).to(DEV).contiguous()
+    out = torch.empty((n, H * DV), dtype=torch.bfloat16, device=DEV)
+    counts = [T - f for T, f in zip(lens, firsts)]
+    cu = torch.tensor([0, counts[0], n], dtype=torch.int32, device=DEV)
+    ws = torch.empty(1 << 26, dtype=torch.uint8, device=DEV)
+    ops.attention(qd, out, cache.to(DEV).unsqueeze(1), None, table.to(DEV), torch.tensor(seq, dtype=torch.int32, device=DEV),
+                  torch.tensor(pos, dtype=torch.int32, device=DEV), H, 1, DK, DK ** -0.5, window, algo=ops.ATTN_MFMA,
+                  workspace=ws, cu_seqlens=cu, max_new=max(counts), q_counts=counts, max_len=max(lens),
+                  v_head_dim=DV, values_in_keys=True)
+    got, ref = out.float().cpu().view(n, H, DV), torch.cat(refs)
+    err = (got - ref).abs().amax(dim=(1, 2))
+    assert float(err.max()) < 2e-2 * max(1.0, float(ref.abs().max())), f"row {int(err.argmax())}, position {pos[int(err.argmax())]}"
