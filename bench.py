@@ -2,6 +2,7 @@
 """Decode and prefill speed of the Qwen3 shapes with random bfloat16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--model qwen3-8b|qwen3-14b|qwen3-32b]
+    python bench.py --design dokulix [--design-size 2b|8b] [--layers N]
 
 The default run is the Qwen3-8B shape.  A step is one decode step of a batch of 8 sequences,
 each with a 2,048-token random prompt in the cache (context length 4,096): the engine's step
@@ -18,6 +19,13 @@ the wall time of prompt steps of 17, 64 and 256 tokens (``prefill_short_*_ms``);
 decode steps, ``--model qwen3-32b`` 32 prompts of 8,192 tokens with 256 decode steps: ``value``
 is then decoded tokens per second over all decode steps of that workload, ``prefill`` the
 prompt step of the whole batch, and ``--steps`` / ``--warmup`` only bound the decode steps.
+
+``--design dokulix`` leaves the default workload alone and measures another architecture beside
+its closest Qwen3 shape: a Dokulix model of ``--layers`` layers (biased block attention and latent
+attention in turn, relu-gated feed-forward) and a Qwen3 model of the same width, heads, head size,
+feed-forward and number of layers, both with random weights; for each the throughput of a
+2,048-token prompt step and of decode steps of a batch of 8 over 2,048-token prompts, and per kind
+of launch its time against its analytical minimum (``efficiency``), from launch-by-launch timing.
 
 The workloads follow the reference's bench (rocml-cli/src/cmd_bench.rs:79-243): synthetic
 prompts, greedy, no stop token, warm-up first; times are taken around synchronised steps.
@@ -37,6 +45,112 @@ LONG_PROMPT = 32768
 WORKLOADS = {"qwen3-14b": (16, 128, 4096, 128), "qwen3-32b": (32, 8192, 8192, 256)}
 
 
+# layer sizes for --design: width, feed-forward, heads, key/value heads, head size; the latent attention's
+# ranks, rotated part, window; the block attention's block; vocabulary
+DESIGN_SIZES = {
+    "2b": dict(width=2048, ff=6144, heads=16, kv_heads=8, dim=128, q_rank=768, kv_rank=512, rot_dim=64,
+               window=1024, chunk=1024, vocab=32768),
+    "8b": dict(width=4096, ff=12288, heads=32, kv_heads=8, dim=128, q_rank=1536, kv_rank=512, rot_dim=64,
+               window=1024, chunk=1024, vocab=32768),
+}
+
+
+def design_configs(size: dict, n_layers: int):
+    """config.json of the Dokulix model and of the Qwen3 model of equal size."""
+    z = size
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+           "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                     "mask": {"size": z["chunk"]}, "scale": z["dim"] ** -0.5}}
+    lat = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+           "mixer": {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot_dim"], "vdim": z["dim"],
+                     "q_rank": z["q_rank"], "kv_rank": z["kv_rank"], "mask": {"size": z["window"]},
+                     "rot": {"base": 10000.0, "dims": z["rot_dim"]}, "scale": (z["dim"] + z["rot_dim"]) ** -0.5}}
+    dokulix = {"architecture": "Dokulix", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+               "layers": [att if i % 2 == 0 else lat for i in range(n_layers)], "max_positions": 40960}
+    qwen = {"architectures": ["Qwen3ForCausalLM"], "model_type": "qwen3", "vocab_size": z["vocab"],
+            "hidden_size": z["width"], "intermediate_size": z["ff"], "num_hidden_layers": n_layers,
+            "num_attention_heads": z["heads"], "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
+            "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
+            "max_position_embeddings": 40960, "hidden_act": "silu", "attention_bias": False}
+    return dokulix, qwen
+
+
+def run_design(args) -> int:
+    """Prefill and decode throughput of the design beside its closest Qwen3 shape, and every kind of
+    launch against its analytical minimum."""
+    import numpy as np
+    import torch
+    from rocml_amd import ops
+    from rocml_amd.engine import Engine, EngineBackend, Generator, Request, StepEntry
+    from rocml_amd.profile import OpProfiler
+    from rocml_amd.sampling import SamplingParams
+    from rocml_amd.weights import random_model
+
+    ops.load_all()
+    n_layers = args.layers or 4
+    batch = args.batch or 8
+    steps, warmup = max(1, min(args.steps, 64)), min(args.warmup, 8)
+    rng = np.random.default_rng(0)
+    dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    results = {}
+    for name, raw in zip((args.design, "qwen3"), design_configs(DESIGN_SIZES[args.design_size], n_layers)):
+        model = random_model(raw, seed=0, dtype=args.dtype, device="cuda:0")
+        vocab = model.spec.vocab
+        engine = Engine(model, max_tokens=batch * CONTEXT, max_seqs=batch, max_step_tokens=8192)
+
+        def tokens(n):
+            return [int(t) for t in rng.integers(0, vocab, size=n)]
+
+        def prompt_step():
+            slot = engine.new_sequence()
+            toks = tokens(PROMPT_LEN)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            engine.step([StepEntry(slot, toks, [PROMPT_LEN - 1])])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            engine.release(slot)
+            return dt
+
+        prompt_step()
+        prefill_s = sorted(prompt_step() for _ in range(max(1, args.prefill_runs)))[max(1, args.prefill_runs) // 2]
+        gen = Generator(EngineBackend(engine), max_batch=batch)
+        marks = {}
+
+        def on_step(k):
+            if k == warmup or k == warmup + steps:
+                torch.cuda.synchronize()
+                marks[k] = time.perf_counter()
+        gen.on_step = on_step
+        gen.run([Request(tokens(PROMPT_LEN), warmup + steps + 1, SamplingParams.greedy()) for _ in range(batch)])
+        decode_s = (marks[warmup + steps] - marks[warmup]) / steps
+        # launch by launch, with bytes and operations: a prompt step and a few decode steps
+        with OpProfiler(dtype) as prof:
+            gen = Generator(EngineBackend(engine), max_batch=batch)
+            gen.run([Request(tokens(PROMPT_LEN), 5, SamplingParams.greedy()) for _ in range(batch)])
+        report = prof.finish()
+        rows = {ph.phase: {r.label: {"ms": round(r.elapsed_ms, 3), "calls": r.count, "t_min_ms": round(r.t_min_ms, 3),
+                                     "efficiency": round(r.efficiency, 3)} for r in ph.by_op} for ph in report.phases}
+        results[name] = {"prefill_tok_s": round(PROMPT_LEN / prefill_s, 1), "prefill_ms": round(prefill_s * 1e3, 3),
+                         "decode_tok_s": round(batch / decode_s, 1), "decode_ms_per_step": round(decode_s * 1e3, 4),
+                         "params_m": round(model.n_params() / 1e6, 1), "launches": rows}
+        del engine, model, gen
+        torch.cuda.empty_cache()
+    mine, other = results[args.design], results["qwen3"]
+    out = {"metric": f"{args.design} beside the Qwen3 shape of equal size ({args.design_size}, {n_layers} layers, "
+                     f"{args.dtype}): decode tok/s at batch {batch} over {PROMPT_LEN}-token prompts",
+           "value": mine["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+           "ms_per_step": mine["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+           "data": "synthetic: uniform random token ids, random N(0, 0.02) weights",
+           "config": dict(DESIGN_SIZES[args.design_size], layers=n_layers, global_batch=batch, prompt_len=PROMPT_LEN),
+           "decode_vs_qwen3": round(mine["decode_tok_s"] / other["decode_tok_s"], 3),
+           "prefill_vs_qwen3": round(mine["prefill_tok_s"] / other["prefill_tok_s"], 3),
+           args.design: mine, "qwen3": other}
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -48,6 +162,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the further points")
     ap.add_argument("--prefill-runs", type=int, default=3)
+    ap.add_argument("--design", default=None, choices=["dokulix"],
+                    help="measure this architecture at real layer sizes beside the closest Qwen3 shape, instead of the default workload")
+    ap.add_argument("--design-size", default="2b", choices=sorted(DESIGN_SIZES), help="layer sizes for --design")
     ap.add_argument("--skip-prompts", action="store_true",
                     help="profiling aid: give the sequences their 2,048 positions without running the "
                          "prompts (the cache holds zeros); the timed decode steps are the same")
@@ -55,6 +172,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this library")
         return 2
+    if args.design is not None:
+        return run_design(args)
 
     import numpy as np
     import torch

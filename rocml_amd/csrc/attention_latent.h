@@ -25,11 +25,21 @@
 constexpr int AL_ROWS = 64;           // rows of a block
 constexpr int AL_KEYS = 32;           // keys of a piece
 constexpr int AL_VROW = AL_KEYS + 8;  // bf16 per row of the transposed piece (16 bytes of padding)
+constexpr float AL_LAZY_MAX = 8.0f;   // how far a row's maximum may run ahead of its exponents' reference (powers of two)
+
+// Where the transposed piece keeps number d of the keys (bf16 units): rows of AL_VROW and 32 more
+// after every eight rows, so that rows eight apart, which neighbouring groups of lanes write at
+// the same time, lie 16 banks apart.
+__device__ __forceinline__ int al_vrow_at(int d) { return d * AL_VROW + (d >> 3) * 32; }
+
+// Where the piece keeps key k as a row: the first product's tile u reads key 8 (c / 4) + 4 u + c % 4
+// in lane column c; stored at row 16 u + c, the 16 lanes of a tile read 16 consecutive rows.
+__device__ __forceinline__ int al_krow_at(int k) { return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3); }
 
 template <int KD, int DT>
 struct LatentLds {
     static constexpr int K_ROW = KD * 32 + 8;                               // bf16 per key row
-    static constexpr int BYTES = (AL_KEYS * K_ROW + DT * 16 * AL_VROW) * 2;
+    static constexpr int BYTES = (AL_KEYS * K_ROW + DT * 16 * AL_VROW + DT * 2 * 32) * 2;
 };
 
 template <int KD, int DT>
@@ -42,7 +52,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     using L = LatentLds<KD, DT>;
     extern __shared__ uint4 al_smem[];
     bf16_t* sk = (bf16_t*)al_smem;                    // [AL_KEYS][K_ROW]
-    bf16_t* sv = sk + AL_KEYS * L::K_ROW;             // [DT * 16][AL_VROW]
+    bf16_t* sv = sk + AL_KEYS * L::K_ROW;             // [DT * 16] rows at al_vrow_at
     int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int g = lane >> 4, col = lane & 15;
     int split = blockIdx.y;
@@ -105,7 +115,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         for (int i = 0; i < MAX_ITEMS; ++i) {
             int w = tid + i * 256;
             if (w < items) {
-                int kp = w / dk8, dc = w - kp * dk8;
+                int kp = w & 15, dc = w >> 4;           // 16 neighbouring lanes: the 16 pairs of keys, the same 8 numbers
                 ra[i] = *(const uint4*)(base + (size_t)(2 * kp) * dk + dc * 8);
                 rb[i] = *(const uint4*)(base + (size_t)(2 * kp + 1) * dk + dc * 8);
             }
@@ -116,13 +126,13 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         for (int i = 0; i < MAX_ITEMS; ++i) {
             int w = tid + i * 256;
             if (w < items) {
-                int kp = w / dk8, dc = w - kp * dk8;
-                *(uint4*)(sk + (2 * kp) * L::K_ROW + dc * 8) = ra[i];
-                *(uint4*)(sk + (2 * kp + 1) * L::K_ROW + dc * 8) = rb[i];
+                int kp = w & 15, dc = w >> 4;
+                *(uint4*)(sk + al_krow_at(2 * kp) * L::K_ROW + dc * 8) = ra[i];
+                *(uint4*)(sk + al_krow_at(2 * kp + 1) * L::K_ROW + dc * 8) = rb[i];
                 if (dc < dv8) {
                     const uint32_t a[4] = {ra[i].x, ra[i].y, ra[i].z, ra[i].w};
                     const uint32_t c[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
-                    uint32_t* dst = (uint32_t*)(sv + (dc * 8) * AL_VROW + 2 * kp);
+                    uint32_t* dst = (uint32_t*)(sv + al_vrow_at(dc * 8) + 2 * kp);
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         // numbers 2j and 2j + 1 of both keys: (key 2kp, key 2kp + 1) side by side
@@ -149,7 +159,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            const bf16_t* krow = sk + (8 * (col >> 2) + 4 * u + (col & 3)) * L::K_ROW + g * 8;
+            const bf16_t* krow = sk + (16 * u + col) * L::K_ROW + g * 8;       // key 8 (col / 4) + 4 u + col % 4
 #pragma unroll
             for (int kd = 0; kd < KD; ++kd) {
                 bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kd * 32));
@@ -168,9 +178,19 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
             }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        float m_new = fmaxf(m, mx);
-        float m_use = m_new == -INFINITY ? 0.f : m_new;
-        float corr = fast_exp2(m - m_use);
+        // The exponents' reference m follows a row's maximum only when that has grown by more than
+        // AL_LAZY_MAX: any reference gives the same quotient at the end, the probabilities stay below
+        // 2^AL_LAZY_MAX, and the sums and outputs so far are rescaled only for a row's first pieces
+        // instead of with every piece (the outputs are the bulk of a lane's registers).
+        if (__builtin_amdgcn_ballot_w64(mx > m + AL_LAZY_MAX)) {
+            float m_new = fmaxf(m, mx);
+            float corr = fast_exp2(m - (m_new == -INFINITY ? 0.f : m_new));
+            l *= corr;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o[dt] = o[dt] * corr;
+            m = m_new;
+        }
+        float m_use = m == -INFINITY ? 0.f : m;
         float sum = 0.f;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -181,15 +201,13 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
             }
         sum += __shfl_xor(sum, 16, 64);
         sum += __shfl_xor(sum, 32, 64);
-        l = l * corr + sum;
-        m = m_new;
+        l += sum;
         // P^T operand: slots 0..7 = keys 8g .. 8g+7
         bf16x8_t pf = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(s[0][0], s[0][1]), pack_bf16x2(s[0][2], s[0][3]),
                                                               pack_bf16x2(s[1][0], s[1][1]), pack_bf16x2(s[1][2], s[1][3])));
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sv + (dt * 16 + col) * AL_VROW + g * 8));
-            o[dt] = o[dt] * corr;
+            bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sv + al_vrow_at(dt * 16 + col) + g * 8));
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
         }
     }

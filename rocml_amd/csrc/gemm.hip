@@ -617,18 +617,38 @@ ROCML_EXPORT int rocml_gemm(const void* x, int x_dtype, int ldx, const void* w, 
     return 0;
 }
 
+#include "gemm_heads.h"
+
 // A batch of small products that share their shapes: out_b[M, N] = x_b[M, K] * w_b[N, K]^T for
 // b = 0 .. batch-1, operands and results `batch_*` elements apart (the heads of a layer: x and out
 // are column ranges of wider matrices, w is [batch, N, K]).  32-bit accumulation by fused
 // multiply-add in K order for every type; x may be 32-bit while w is bfloat16.
+// gate (may be null): 32-bit [M, ldg] with the heads side by side, batch_g apart: out = product * sigmoid(gate).
 ROCML_EXPORT int rocml_gemm_batched(const void* x, int x_dtype, int ldx, long long batch_x, const void* w, int w_dtype,
                                     int ldw, long long batch_w, void* out, int out_dtype, int ldo, long long batch_o,
-                                    int batch, int m, int n, int k, hipStream_t stream) {
+                                    int batch, int m, int n, int k, const float* gate, int ldg, long long batch_g,
+                                    hipStream_t stream) {
     ROCML_REQUIRE(batch > 0 && batch < 65536 && m >= 0 && n > 0 && k > 0, "gemm_batched: bad sizes batch=%d M=%d N=%d K=%d", batch, m, n, k);
     ROCML_REQUIRE(ldx >= k && ldw >= k && ldo >= n && batch_x >= 0 && batch_w >= 0 && batch_o >= 0,
                   "gemm_batched: row strides (%d, %d, %d) below (K, K, N) or a negative batch stride", ldx, ldw, ldo);
     ROCML_REQUIRE(ceil_div(m, GT_BM) < 65536, "gemm_batched: too many rows %d", m);
+    ROCML_REQUIRE(!gate || ldg >= n, "gemm_batched: gate rows of %d numbers for N=%d", ldg, n);
     if (m == 0) return 0;
+    // The matrix cores: bfloat16 weights [batch, N, K] without gaps, operands that 16-byte loads reach.
+    int x_align = x_dtype == ROCML_F32 ? 4 : 8;
+    bool mfma = w_dtype == ROCML_BF16 && out_dtype == ROCML_BF16 && ldw == k && batch_w == (long long)n * k && k % 8 == 0 &&
+                ldx % x_align == 0 && batch_x % x_align == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
+    if (mfma) {
+        dim3 grid(ceil_div(n, GH_BN), ceil_div(m, GH_BM), batch);
+#define GH(TX, G) gemm_heads_mfma_kernel<TX, bf16_t, G><<<grid, 256, 0, stream>>>(                       \
+        (const TX*)x, ldx, (int)batch_x, (const bf16_t*)w, (bf16_t*)out, ldo, (int)batch_o, m, n, k, gate, ldg, (int)batch_g)
+        if (x_dtype == ROCML_F32) { if (gate) GH(float, true); else GH(float, false); }
+        else { if (gate) GH(bf16_t, true); else GH(bf16_t, false); }
+#undef GH
+        ROCML_CHECK_LAUNCH("gemm_batched");
+        return 0;
+    }
+    ROCML_REQUIRE(!gate, "gemm_batched: the gate goes with the matrix-core kernel (bfloat16 weights and output, K a multiple of 8)");
 #define GB(TX, TW, TO) launch_gemm_tile_batched<TX, TW, TO>(x, ldx, batch_x, w, ldw, batch_w, out, ldo, batch_o, batch, m, n, k, stream)
     if (x_dtype == ROCML_F32 && w_dtype == ROCML_F32 && out_dtype == ROCML_F32) GB(float, float, float);
     else if (x_dtype == ROCML_F32 && w_dtype == ROCML_BF16 && out_dtype == ROCML_BF16) GB(float, bf16_t, bf16_t);

@@ -42,7 +42,7 @@ _SIGNATURES = {
     "gemm": {
         "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _LL, _P, _I, _F, _I, _P],
         "rocml_splitk_reduce": [_P, _P, _I, _I, _I, _I, _I, _I, _P],
-        "rocml_gemm_batched": [_P, _I, _I, _LL, _P, _I, _I, _LL, _P, _I, _I, _LL, _I, _I, _I, _I, _P],
+        "rocml_gemm_batched": [_P, _I, _I, _LL, _P, _I, _I, _LL, _P, _I, _I, _LL, _I, _I, _I, _I, _P, _I, _LL, _P],
         "rocml_gemm_residual_prescale_pays": [_I, _I, _I],
         "rocml_gemm_residual_prescale": [_P, _I, _P, _I, _P, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P],
     },
@@ -440,11 +440,25 @@ def gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     return deferred.value
 
 
-def gemm_batched(x: torch.Tensor, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_head_stride: int) -> None:
+def gemm_batched_gate_fusable(w: torch.Tensor, x: torch.Tensor) -> bool:
+    """Whether ``gemm_batched`` can apply an output gate itself (its matrix-core kernel runs)."""
+    return (w.dtype == torch.bfloat16 and w.shape[2] % 8 == 0 and x.shape[1] % (4 if x.dtype == torch.float32 else 8) == 0)
+
+
+def gemm_batched(x: torch.Tensor, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_head_stride: int,
+                 gate: Optional[torch.Tensor] = None) -> None:
     """One small product per head: ``out[:, h * out_head_stride : ... + N] = x[:, h * x_head_stride :
     ... + K] @ w[h].T`` for ``w [heads, N, K]``; ``x`` and ``out`` are ``[tokens, width]`` matrices
-    that hold the heads side by side.  32-bit accumulation; ``x`` may be 32-bit with bfloat16 weights."""
+    that hold the heads side by side.  32-bit accumulation; ``x`` may be 32-bit with bfloat16 weights.
+    ``gate`` (32-bit ``[tokens, heads * N]``, rows may be a column range of a wider matrix): the
+    product is multiplied by ``sigmoid(gate)``; only where ``gemm_batched_gate_fusable``."""
     _dev(x, w, out)
+    ldg = g_stride = 0
+    if gate is not None:
+        if not gate.is_cuda or gate.dtype != torch.float32 or gate.stride(1) != 1 or gate.shape != (x.shape[0], w.shape[0] * w.shape[1]) \
+                or out_head_stride != w.shape[1] or not gemm_batched_gate_fusable(w, x) or x_head_stride % 4:
+            raise KernelError("the gate must be 32-bit [tokens, heads * N] for an output without gaps, on the matrix-core kernel")
+        ldg, g_stride = (gate.stride(0) if x.shape[0] > 1 else max(gate.stride(0), gate.shape[1])), w.shape[1]
     if x.dim() != 2 or out.dim() != 2 or w.dim() != 3 or x.shape[0] != out.shape[0]:
         raise KernelError("gemm_batched takes x [T, width], w [heads, N, K], out [T, width]")
     heads, n, k = w.shape
@@ -452,7 +466,7 @@ def gemm_batched(x: torch.Tensor, x_head_stride: int, w: torch.Tensor, out: torc
         raise KernelError(f"{heads} heads of K={k} / N={n} do not fit rows of {x.shape[1]} / {out.shape[1]}")
     _check("gemm", library("gemm").rocml_gemm_batched(
         _ptr(x), _code(x), x.shape[1], x_head_stride, _ptr(w), _code(w), k, n * k, _ptr(out), _code(out),
-        out.shape[1], out_head_stride, heads, x.shape[0], n, k, _stream()))
+        out.shape[1], out_head_stride, heads, x.shape[0], n, k, _ptr(gate), ldg, g_stride, _stream()))
 
 
 PRESCALE_MAX_ROWS = 16      # most rows gemm_residual_prescale takes

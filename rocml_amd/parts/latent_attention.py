@@ -17,8 +17,8 @@ Both small products run once per token and head, whatever the number of keys.
 Launches of a step: one product for the three projections of ``h`` (query latent, key/value
 latent with its rotated part, output gate), one kernel that norms both latents, rotates and
 appends to the cache, the product ``W_uq``, the rotation of the queries' rotated parts, the
-per-head products with ``W_uk^T``, the attention, the per-head products with ``W_uv``, the gate,
-and the output product whose epilogue is the residual sum.
+per-head products with ``W_uk^T``, the attention, the per-head products with ``W_uv`` (the gate is
+their epilogue in bfloat16), and the output product whose epilogue is the residual sum.
 """
 from __future__ import annotations
 
@@ -140,9 +140,13 @@ class LatentAttention(Mixer):
                       cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
                       max_len=step.max_len, v_head_dim=s.kv_rank, values_in_keys=True)
         o = ws.get("latent.o", (n, self.o_dim), self.dtype)
-        ops.gemm_batched(ol, s.kv_rank, self.w_uv, o, s.v_head_dim)
-        if s.gate:
-            ops.sigmoid_gate(o, first[:, s.q_rank + self.row:])
+        gate = first[:, s.q_rank + self.row:] if s.gate else None
+        if gate is not None and ops.gemm_batched_gate_fusable(self.w_uv, ol) and s.kv_rank % 8 == 0:
+            ops.gemm_batched(ol, s.kv_rank, self.w_uv, o, s.v_head_dim, gate=gate)      # the gate is the product's epilogue
+        else:
+            ops.gemm_batched(ol, s.kv_rank, self.w_uv, o, s.v_head_dim)
+            if gate is not None:
+                ops.sigmoid_gate(o, gate)
         stream(step).add_product(o, self.w_o, x_accum)
 
 

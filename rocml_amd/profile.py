@@ -48,12 +48,28 @@ def _gemm_cost(x, w, out, *a, **kw) -> Tuple[int, int]:
 
 
 def _attention_cost(q, out, k_cache, v_cache, block_table, token_seq, token_pos, n_heads, n_kv_heads, head_dim,
-                    *a, **kw) -> Tuple[int, int]:
+                    scale=None, window=None, *a, **kw) -> Tuple[int, int]:
     n_tokens, max_new, max_len = q.shape[0], kw.get("max_new", 0), kw.get("max_len", 0)
     n_seqs = block_table.shape[0]
-    kv = 2 * n_seqs * max_len * n_kv_heads * head_dim * k_cache.element_size()
+    dv = kw.get("v_head_dim") or head_dim
+    row = head_dim if kw.get("values_in_keys") else head_dim + dv           # numbers read per key and key/value head
     keys_per_query = max_len if max_new <= 1 else max(1, max_len - max_new // 2)     # causal: half of the new part
-    return _nbytes(q, out) + kv, 4 * n_heads * head_dim * n_tokens * keys_per_query
+    read_len = max_len
+    if kw.get("chunk"):                      # a query sees its own block up to itself: half a block on average
+        keys_per_query = min(keys_per_query, max(1, kw["chunk"] // 2))
+        read_len = min(max_len, max_new + kw["chunk"])
+    elif window:
+        keys_per_query = min(keys_per_query, window)
+        read_len = min(max_len, max_new + window)
+    kv = n_seqs * read_len * n_kv_heads * row * k_cache.element_size()
+    return _nbytes(q, out) + kv, 2 * n_heads * (head_dim + dv) * n_tokens * keys_per_query
+
+
+def _gemm_batched_cost(x, x_head_stride, w, out, out_head_stride, **kw) -> Tuple[int, int]:
+    heads, n, k = w.shape
+    rows = x.shape[0]
+    moved = rows * heads * (k * x.element_size() + n * out.element_size()) + _nbytes(w)
+    return moved, 2 * rows * heads * n * k
 
 
 def _fused_attention_cost(qkv, out, k_cache, v_cache, block_table, token_seq, token_pos, n_heads, n_kv_heads, head_dim,
@@ -86,7 +102,9 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
     "gemm": ("product", _gemm_cost),
     "gemm_residual_prescale": ("product", lambda x, w, resid, gain, xg, ssq, *a, **kw: (
         _nbytes(x, w, resid, resid, gain, xg, ssq), 2 * x.shape[0] * w.shape[0] * x.shape[1])),
-    "attention": ("attention", _attention_cost),
+    "attention": (lambda *a, **kw: "attention over latent rows" if kw.get("values_in_keys") else
+                  "attention (blocks, slopes, sink)" if kw.get("chunk") or kw.get("sink") or kw.get("slopes") is not None
+                  else "attention", _attention_cost),
     "attention_decode_fused": ("attention (norm, rotation, append)", _fused_attention_cost),
     "attention_prefill_fused": ("attention (query norm, rotation)", _prefill_fused_cost),
     "qk_norm_rope_append": ("q/k norm, rotation, append", _tensor_args_cost(skip=(11, 12))),   # not the whole cache
@@ -95,6 +113,13 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
     "embed_gather": ("embedding", lambda table, ids, out, *a, **kw: (2 * _nbytes(out) + _nbytes(ids), 0)),
     "rope_table": ("rotation table", _tensor_args_cost()),
     "add_into": ("residual add", _tensor_args_cost()),
+    "add_row_vector": ("row vector add", lambda x, b: (2 * _nbytes(x) + _nbytes(b), x.numel())),
+    "gemm_batched": ("per-head products", _gemm_batched_cost),
+    "latent_prepare": ("latent norms, rotation, append", lambda proj, *a, **kw: (
+        proj.shape[0] * sum(a[:3]) * 6, proj.shape[0] * sum(a[:3]) * 4)),
+    "rope_heads": ("rotation of the queries' part", lambda q, n_heads, head_stride, offset, rot_part, *a, **kw: (
+        q.shape[0] * n_heads * rot_part * 6, q.shape[0] * n_heads * rot_part * 3)),
+    "sigmoid_gate": ("output gate", lambda y, gate: (2 * _nbytes(y) + y.numel() * 4, 4 * y.numel())),
     "splitk_reduce": ("sum of K pieces", _tensor_args_cost()),
     "argmax": ("argmax", _tensor_args_cost()),
     "sample": ("sampling", lambda logits, *a, **kw: (_nbytes(logits), 0)),
@@ -191,7 +216,8 @@ class OpProfiler:
             result = fn(*a, **kw)
             end.record()
             b, f = cost(*a, **kw)
-            self._records.append((self.phase, label, int(b), int(f), start, end))
+            name = label(*a, **kw) if callable(label) else label       # (a label may depend on the call)
+            self._records.append((self.phase, name, int(b), int(f), start, end))
             return result
         return timed
 

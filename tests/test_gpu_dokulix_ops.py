@@ -357,3 +357,26 @@ def test_matrix_core_kernel_for_latent_rows(H, DK, DV, window, decode):
     got, ref = out.float().cpu().view(n, H, DV), torch.cat(refs)
     err = (got - ref).abs().amax(dim=(1, 2))
     assert float(err.max()) < 2e-2 * max(1.0, float(ref.abs().max())), f"row {int(err.argmax())}, position {pos[int(err.argmax())]}"
+
+
+@pytest.mark.parametrize("tx", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,H,K,N,xs,os_", [(1, 3, 16, 24, 24, 32), (8, 16, 128, 512, 192, 576), (70, 4, 40, 20, 48, 20),
+                                            (300, 2, 512, 128, 512, 128), (17, 6, 64, 32, 64, 32)])
+def test_per_head_products_on_the_matrix_cores(tx, T, H, K, N, xs, os_):
+    """bfloat16 weights, strides that 16-byte loads reach: the matrix-core kernel; with the gate as its epilogue
+    where the output has no gaps."""
+    from rocml_amd import ops
+    gen = torch.Generator().manual_seed(T + K + N)
+    x = torch.randn(T, H * xs, generator=gen).to(tx)
+    w = (torch.randn(H, N, K, generator=gen) * K ** -0.5).to(torch.bfloat16)
+    ref = torch.einsum("thk,hnk->thn", x.float().view(T, H, xs)[..., :K], w.float())
+    gate = torch.randn(T, 7 + H * N, generator=gen)
+    for use_gate in (False, True):
+        if use_gate and os_ != N:
+            continue
+        out = torch.zeros((T, H * os_), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_batched(x.to(DEV), xs, w.to(DEV), out, os_, gate=gate.to(DEV)[:, 7:] if use_gate else None)
+        want = ref * torch.sigmoid(gate[:, 7:].view(T, H, N)) if use_gate else ref
+        got = out.float().cpu().view(T, H, os_)
+        assert float((got[..., :N] - want).abs().max()) < 1.5e-2 * float(want.abs().max())
+        assert os_ == N or float(got[..., N:].abs().max()) == 0.0
