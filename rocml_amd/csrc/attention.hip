@@ -153,12 +153,13 @@ static int launch_latent(const LatentArgs& a, hipStream_t stream) {
         if (allow_lds(attn_latent_mfma_kernel<KD, DT>, L::BYTES)) return 1;
         ready = true;
     }
-    // Splits of the key range: enough blocks for two a CU, at most one per piece the rows can see.
+    // Splits of the key range: enough blocks for one a CU, at most one per two pieces the rows can see
+    // (a block's first piece costs it four trips to memory, a further one about one).
     // The choice follows the launch's shape (rows, window, width of the block table), not the lengths.
     int cus = cu_count();
     int pieces = a.window > 0 ? a.window / AL_KEYS + 2 : a.bt_width * (AM_PAGE / AL_KEYS);
-    int n_splits = 2 * cus / a.tiles;
-    if (n_splits > pieces) n_splits = pieces;
+    int n_splits = cus / a.tiles;
+    if (n_splits > (pieces + 1) / 2) n_splits = (pieces + 1) / 2;
     if (n_splits > 64) n_splits = 64;
     long long rows = (long long)a.n_tokens * a.n_heads;
     long long per_split = rows * (a.dv + 2) * (long long)sizeof(float);
@@ -170,7 +171,7 @@ static int launch_latent(const LatentArgs& a, hipStream_t stream) {
         a.q, a.out, a.cache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos, a.n_heads, a.dk, a.dv,
         a.scale * LOG2E, a.window, n_splits, part_o, part_ml);
     if (n_splits > 1)
-        attn_latent_reduce_kernel<<<(unsigned)rows, a.dv >= 256 ? 256 : 128, 0, stream>>>(part_o, part_ml, a.out, n_splits, a.dv);
+        attn_latent_reduce_kernel<<<(unsigned)rows, a.dv > 256 ? 256 : a.dv > 128 ? 128 : 64, 0, stream>>>(part_o, part_ml, a.out, n_splits, a.dv);
     return 0;
 }
 

@@ -237,22 +237,33 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     }
 }
 
-// Log-sum-exp merge of the splits of a row, in split order; one block per row, a thread per number.
+// Log-sum-exp merge of the splits of a row, in split order: one block per row.  At most 64 splits:
+// lane s of every wave fetches split s's reference and sum, so these loads go out together; the
+// weights then sit in LDS and every thread sums its numbers over the splits, eight loads at a time.
 __global__ void attn_latent_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                           bf16_t* __restrict__ out, int n_splits, int dv) {
+    __shared__ float wgt[64];
     size_t row = blockIdx.x;
     const float* ml = part_ml + row * n_splits * 2;
-    float mm = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, ml[s * 2]);
-    float ll = 0.f;
-    for (int s = 0; s < n_splits; ++s) ll += ml[s * 2] == -INFINITY ? 0.f : ml[s * 2 + 1] * fast_exp2(ml[s * 2] - mm);
-    float inv = 1.0f / ll;
+    const float* po = part_o + row * n_splits * dv;
+    int lane = threadIdx.x & 63;
+    bool has = lane < n_splits;
+    float ms = has ? ml[lane * 2] : -INFINITY;
+    float ls = has ? ml[lane * 2 + 1] : 0.f;
+    float mm = wave_max(ms);
+    float w = ms == -INFINITY ? 0.f : fast_exp2(ms - mm);
+    if (threadIdx.x < 64) wgt[lane] = w;
+    float inv_l = 1.0f / wave_sum(ls * w);          // every wave computes the same sum
+    __syncthreads();
     for (int d = threadIdx.x; d < dv; d += blockDim.x) {
         float acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            float w = ml[s * 2] == -INFINITY ? 0.f : fast_exp2(ml[s * 2] - mm);
-            acc += part_o[(row * n_splits + s) * dv + d] * w;
+        for (int s0 = 0; s0 < n_splits; s0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int s = 0; s < 8; ++s) v[s] = po[(size_t)min(s0 + s, n_splits - 1) * dv + d];
+#pragma unroll
+            for (int s = 0; s < 8; ++s) acc += s0 + s < n_splits ? v[s] * wgt[s0 + s] : 0.f;
         }
-        out[row * dv + d] = f32_to_bf16(acc * inv);
+        out[row * dv + d] = f32_to_bf16(acc * inv_l);
     }
 }

@@ -639,11 +639,15 @@ ROCML_EXPORT int rocml_gemm_batched(const void* x, int x_dtype, int ldx, long lo
     bool mfma = w_dtype == ROCML_BF16 && out_dtype == ROCML_BF16 && ldw == k && batch_w == (long long)n * k && k % 8 == 0 &&
                 ldx % x_align == 0 && batch_x % x_align == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0;
     if (mfma) {
-        dim3 grid(ceil_div(n, GH_BN), ceil_div(m, GH_BM), batch);
-#define GH(TX, G) gemm_heads_mfma_kernel<TX, bf16_t, G><<<grid, 256, 0, stream>>>(                       \
-        (const TX*)x, ldx, (int)batch_x, (const bf16_t*)w, (bf16_t*)out, ldo, (int)batch_o, m, n, k, gate, ldg, (int)batch_g)
-        if (x_dtype == ROCML_F32) { if (gate) GH(float, true); else GH(float, false); }
-        else { if (gate) GH(bf16_t, true); else GH(bf16_t, false); }
+        bool few = m <= 16;
+        dim3 grid(few ? ceil_div(n, 32) : ceil_div(n, GH_BN), few ? 1 : ceil_div(m, GH_BM), batch);
+#define GH(TX, G)                                                                                        \
+        if (few) gemm_heads_few_rows_kernel<TX, bf16_t, G><<<grid, 256, 0, stream>>>(                    \
+            (const TX*)x, ldx, (int)batch_x, (const bf16_t*)w, (bf16_t*)out, ldo, (int)batch_o, m, n, k, gate, ldg, (int)batch_g); \
+        else gemm_heads_mfma_kernel<TX, bf16_t, G><<<grid, 256, 0, stream>>>(                            \
+            (const TX*)x, ldx, (int)batch_x, (const bf16_t*)w, (bf16_t*)out, ldo, (int)batch_o, m, n, k, gate, ldg, (int)batch_g)
+        if (x_dtype == ROCML_F32) { if (gate) { GH(float, true); } else { GH(float, false); } }
+        else { if (gate) { GH(bf16_t, true); } else { GH(bf16_t, false); } }
 #undef GH
         ROCML_CHECK_LAUNCH("gemm_batched");
         return 0;
