@@ -183,6 +183,8 @@ def _describe(spec) -> str:
     """A part's spec in a few words: its kind and its sizes (the width it shares with the model
     left out)."""
     import dataclasses
+    if spec is None:
+        return "none"
     if not dataclasses.is_dataclass(spec):
         return getattr(spec, "kind", type(spec).__name__)
     fields = [f"{f.name}={getattr(spec, f.name)}" for f in dataclasses.fields(spec)
@@ -225,7 +227,7 @@ def cmd_init(args) -> int:
 
 
 def build_parser() -> argparse.ArgumentParser:
-    ap = argparse.ArgumentParser(prog="rocml_amd", description="Qwen3 generation on one MI355X")
+    ap = argparse.ArgumentParser(prog="rocml_amd", description="generation with the decoders of this library on one MI355X")
     sub = ap.add_subparsers(dest="command", required=True)
     g = sub.add_parser("generate", help="continue prompts")
     _add_model_args(g)

@@ -64,6 +64,31 @@ CATALOG: List[ModelEntry] = [
                sampling=QWEN_THINKING_SAMPLING),
 ]
 
+
+
+def _dokulix(vocab, width, ff, heads, kv_heads, dim, q_rank, kv_rank, rot_dim, window, chunk, n_layers, loop=None):
+    """A Dokulix configuration whose layers are block attention and latent attention in turn."""
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "mask": {"size": chunk},
+                     "scale": dim ** -0.5}}
+    lat = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": dim, "q_rank": q_rank, "kv_rank": kv_rank,
+                     "mask": {"size": window}, "rot": {"base": 10000.0, "dims": rot_dim}, "scale": (dim + rot_dim) ** -0.5}}
+    cfg = {"architecture": "Dokulix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+           "layers": [att if i % 2 == 0 else lat for i in range(n_layers)], "max_positions": 40960}
+    if loop is not None:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
+# The second architecture: a test-sized model whose middle layers run twice, and the layer sizes of a
+# 2B-class model (random weights; no checkpoint of this design exists).
+CATALOG += [
+    ModelEntry("dokulix-tiny", _dokulix(320, 96, 160, 4, 2, 32, 48, 32, 16, 40, 48, 4, loop=(1, 3, 2)),
+               default_ctx=512, init_norm_jitter=True),
+    ModelEntry("dokulix-2b", _dokulix(32768, 2048, 6144, 16, 8, 128, 768, 512, 64, 1024, 1024, 24)),
+]
+
 _BY_NAME = {e.name: e for e in CATALOG}
 
 

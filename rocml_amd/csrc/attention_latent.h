@@ -32,9 +32,12 @@ constexpr float AL_LAZY_MAX = 8.0f;   // how far a row's maximum may run ahead o
 // the same time, lie 16 banks apart.
 __device__ __forceinline__ int al_vrow_at(int d) { return d * AL_VROW + (d >> 3) * 32; }
 
-// Where the piece keeps key k as a row: the first product's tile u reads key 8 (c / 4) + 4 u + c % 4
-// in lane column c; stored at row 16 u + c, the 16 lanes of a tile read 16 consecutive rows.
-__device__ __forceinline__ int al_krow_at(int k) { return 16 * ((k >> 2) & 1) + 4 * (k >> 3) + (k & 3); }
+// Keys as rows: the first product's tile u reads key 8 (c / 4) + 4 u + c % 4 in lane column c; that key
+// is stored at row 16 u + c, so the 16 lanes of a tile read 16 consecutive rows.  A thread that
+// stages the piece takes the two keys of one column c (they are 4 apart) and writes rows c and
+// 16 + c: 16 neighbouring lanes write 16 consecutive rows.  In the transposed copy the two keys
+// stand side by side (key 8 G + 4 u + i at place 8 G + 2 i + u of its row), one 4-byte store; the
+// probabilities are packed in the same order.
 
 template <int KD, int DT>
 struct LatentLds {
@@ -101,8 +104,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
 #pragma unroll
     for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // A piece on its way: a thread takes pairs of keys (2 kp, 2 kp + 1) and 8 numbers of both, so
-    // that the transposed copy is written two keys (4 bytes) at a time.
+    // A piece on its way: a thread takes the two keys of a column (see above) and 8 numbers of both.
     int dk8 = dk / 8, dv8 = dv / 8;
     int items = (AL_KEYS / 2) * dk8;
     constexpr int MAX_ITEMS = (AL_KEYS / 2) * (KD * 4) / 256 + 1;
@@ -115,9 +117,10 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         for (int i = 0; i < MAX_ITEMS; ++i) {
             int w = tid + i * 256;
             if (w < items) {
-                int kp = w & 15, dc = w >> 4;           // 16 neighbouring lanes: the 16 pairs of keys, the same 8 numbers
-                ra[i] = *(const uint4*)(base + (size_t)(2 * kp) * dk + dc * 8);
-                rb[i] = *(const uint4*)(base + (size_t)(2 * kp + 1) * dk + dc * 8);
+                int c = w & 15, dc = w >> 4;            // 16 neighbouring lanes: the 16 columns, the same 8 numbers
+                int ka = 8 * (c >> 2) + (c & 3);
+                ra[i] = *(const uint4*)(base + (size_t)ka * dk + dc * 8);
+                rb[i] = *(const uint4*)(base + (size_t)(ka + 4) * dk + dc * 8);
             }
         }
     };
@@ -126,18 +129,18 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         for (int i = 0; i < MAX_ITEMS; ++i) {
             int w = tid + i * 256;
             if (w < items) {
-                int kp = w & 15, dc = w >> 4;
-                *(uint4*)(sk + al_krow_at(2 * kp) * L::K_ROW + dc * 8) = ra[i];
-                *(uint4*)(sk + al_krow_at(2 * kp + 1) * L::K_ROW + dc * 8) = rb[i];
+                int c = w & 15, dc = w >> 4;
+                *(uint4*)(sk + c * L::K_ROW + dc * 8) = ra[i];
+                *(uint4*)(sk + (16 + c) * L::K_ROW + dc * 8) = rb[i];
                 if (dc < dv8) {
                     const uint32_t a[4] = {ra[i].x, ra[i].y, ra[i].z, ra[i].w};
-                    const uint32_t c[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
-                    uint32_t* dst = (uint32_t*)(sv + al_vrow_at(dc * 8) + 2 * kp);
+                    const uint32_t bw[4] = {rb[i].x, rb[i].y, rb[i].z, rb[i].w};
+                    uint32_t* dst = (uint32_t*)(sv + al_vrow_at(dc * 8) + 2 * c);
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        // numbers 2j and 2j + 1 of both keys: (key 2kp, key 2kp + 1) side by side
-                        dst[(2 * j) * (AL_VROW / 2)] = (a[j] & 0xffffu) | (c[j] << 16);
-                        dst[(2 * j + 1) * (AL_VROW / 2)] = (a[j] >> 16) | (c[j] & 0xffff0000u);
+                        // numbers 2j and 2j + 1 of both keys, the two keys side by side
+                        dst[(2 * j) * (AL_VROW / 2)] = (a[j] & 0xffffu) | (bw[j] << 16);
+                        dst[(2 * j + 1) * (AL_VROW / 2)] = (a[j] >> 16) | (bw[j] & 0xffff0000u);
                     }
                 }
             }
@@ -202,9 +205,9 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         sum += __shfl_xor(sum, 16, 64);
         sum += __shfl_xor(sum, 32, 64);
         l += sum;
-        // P^T operand: slots 0..7 = keys 8g .. 8g+7
-        bf16x8_t pf = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(s[0][0], s[0][1]), pack_bf16x2(s[0][2], s[0][3]),
-                                                              pack_bf16x2(s[1][0], s[1][1]), pack_bf16x2(s[1][2], s[1][3])));
+        // P^T operand: slot 2 i + u = key 8 g + 4 u + i, the order of the transposed copy
+        bf16x8_t pf = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(s[0][0], s[1][0]), pack_bf16x2(s[0][1], s[1][1]),
+                                                              pack_bf16x2(s[0][2], s[1][2]), pack_bf16x2(s[0][3], s[1][3])));
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sv + al_vrow_at(dt * 16 + col) + g * 8));

@@ -85,7 +85,8 @@ def test_schedule_rules():
 def test_catalog_and_resolve(tmp_path):
     assert len(set(catalog_names())) == len(CATALOG)              # names are unique
     for e in CATALOG:
-        Qwen3Config.from_dict(e.config)                            # every entry is a valid configuration
+        arch = architecture_of(e.config)
+        arch.to_spec(arch.read_config(e.config))                   # every entry is a valid configuration of its architecture
     assert resolve("qwen3-8b").entry.config["num_hidden_layers"] == 36
     assert resolve("qwen3-8b").entry.sampling.temperature == pytest.approx(0.6)
     with pytest.raises(UnknownModelError, match="qwen3-8b"):       # lists the known names

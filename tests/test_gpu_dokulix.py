@@ -200,3 +200,17 @@ def test_replay_program(models, tmp_path):
             got = torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{step['step']}.f32"), dtype="<f4").reshape(-1, vocab))
             want = torch.stack([refs[r][i] for r, i in rows])
             assert helpers.per_position(got, want) < tol, f"step {step['step']} in {dtype}"
+
+
+def test_command_line_runs_the_design(models, capsys):
+    from rocml_amd.cli import main
+    path, cfg, tensors = models["P"]
+    prompt = helpers.random_tokens(9, cfg["vocab"], 77)
+    rc = main(["generate", "--model", path, "--dtype", "float32", "--prompt-ids", " ".join(map(str, prompt)),
+               "-n", "6", "--ctx", "128", "--batch", "2"])
+    out = capsys.readouterr().out.strip().splitlines()
+    assert rc == 0 and [int(t) for t in out[-1].split()] == plain.greedy(cfg, tensors, prompt, 6)
+    # a catalog name: random weights, no file
+    assert main(["generate", "--model", "dokulix-tiny", "--prompt-ids", "1 2 3", "-n", "4", "--ctx", "64", "--batch", "1"]) == 0
+    assert len(capsys.readouterr().out.strip().splitlines()[-1].split()) == 4
+    assert main(["models"]) == 0 and "dokulix-2b" in capsys.readouterr().out
