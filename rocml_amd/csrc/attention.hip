@@ -145,12 +145,12 @@ struct LatentArgs {
     float scale; int window; int tiles; void* workspace; long long workspace_bytes;
 };
 
-template <int KD, int DT>
+template <int KD, int DT, int RT>
 static int launch_latent(const LatentArgs& a, hipStream_t stream) {
     using L = LatentLds<KD, DT>;
     static bool ready = false;
     if (!ready) {
-        if (allow_lds(attn_latent_mfma_kernel<KD, DT>, L::BYTES)) return 1;
+        if (allow_lds(attn_latent_mfma_kernel<KD, DT, RT>, L::BYTES)) return 1;
         ready = true;
     }
     // Splits of the key range: enough blocks for one a CU, at most one per two pieces the rows can see
@@ -167,7 +167,7 @@ static int launch_latent(const LatentArgs& a, hipStream_t stream) {
     if (n_splits < 1) n_splits = 1;
     float* part_o = (float*)a.workspace;
     float* part_ml = part_o ? part_o + rows * n_splits * a.dv : nullptr;
-    attn_latent_mfma_kernel<KD, DT><<<dim3(a.tiles, n_splits), 256, L::BYTES, stream>>>(
+    attn_latent_mfma_kernel<KD, DT, RT><<<dim3(a.tiles, n_splits), 256, L::BYTES, stream>>>(
         a.q, a.out, a.cache, a.block_table, a.bt_width, a.cu_seqlens, a.n_seqs, a.token_pos, a.n_heads, a.dk, a.dv,
         a.scale * LOG2E, a.window, n_splits, part_o, part_ml);
     if (n_splits > 1)
@@ -241,16 +241,21 @@ ROCML_EXPORT int rocml_attention(const void* q, void* out, const void* kcache, c
                                  "key/value head, sizes that are multiples of 8 up to 576 and 512, and the sequence offsets "
                                  "(D=%d Dv=%d Hkv=%d)", d, dv, hkv);
     if (latent_ok && algo != ATTN_PLAIN) {
+        // two tiles of rows a wave where the sequences bring at least 128 rows each on average (prompts)
+        // and the sizes leave the registers for it
+        int kd = (d + 31) / 32, dt = (dv + 15) / 16;
+        int rt = (long long)n_tokens * hq >= 128ll * n_seqs && kd <= 10 && dt <= 16 ? 2 : 1;
         long long tiles = 0;
-        for (int b = 0; b < n_seqs; ++b) tiles += ((long long)q_counts[b] * hq + AL_ROWS - 1) / AL_ROWS;
+        for (int b = 0; b < n_seqs; ++b) tiles += ((long long)q_counts[b] * hq + AL_ROWS * rt - 1) / (AL_ROWS * rt);
         ROCML_REQUIRE(tiles > 0 && tiles < (1ll << 31), "attention: %lld row tiles", tiles);
         LatentArgs a{(const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kcache, block_table, bt_width, cu_seqlens, n_seqs,
                      token_pos, n_tokens, hq, d, dv, scale, window, (int)tiles, workspace, workspace_bytes};
-        int kd = (d + 31) / 32, dt = (dv + 15) / 16;
-        int rc = kd <= 3 && dt <= 4     ? launch_latent<3, 4>(a, stream)
-                 : kd <= 6 && dt <= 8   ? launch_latent<6, 8>(a, stream)
-                 : kd <= 10 && dt <= 16 ? launch_latent<10, 16>(a, stream)
-                                        : launch_latent<18, 32>(a, stream);
+#define BY_ROW_TILES(KD_, DT_) (rt == 2 ? launch_latent<KD_, DT_, 2>(a, stream) : launch_latent<KD_, DT_, 1>(a, stream))
+        int rc = kd <= 3 && dt <= 4     ? BY_ROW_TILES(3, 4)
+                 : kd <= 6 && dt <= 8   ? BY_ROW_TILES(6, 8)
+                 : kd <= 10 && dt <= 16 ? BY_ROW_TILES(10, 16)
+                                        : launch_latent<18, 32, 1>(a, stream);
+#undef BY_ROW_TILES
         if (rc) return rc;
         ROCML_CHECK_LAUNCH("attention over latent rows");
         return 0;

@@ -7,8 +7,11 @@
 //
 // Rows of work are the (token, head) pairs of a step: the queries [T, H, DK] and the outputs
 // [T, H, DV] are plain matrices of T * H rows, and row r of a sequence's new tokens stands at
-// position pos0 + r / H.  A block takes 64 consecutive rows of one sequence (16 per wave: the 16
-// columns of an MFMA) and one split of their keys; keys come 32 at a time through LDS, once as
+// position pos0 + r / H.  A block takes 64 RT consecutive rows of one sequence (RT tiles of 16 per
+// wave: the 16 columns of an MFMA; RT = 2 for prompts, where every key operand read from LDS then
+// feeds two products and a loaded key serves 128 rows, RT = 1 for the few rows of a decode step and
+// for the widest sizes, whose two tiles of outputs and queries would not fit a lane's 512 registers)
+// and one split of their keys; keys come 32 at a time through LDS, once as
 // rows (the first product, S^T = K Q^T, reads 8 numbers of a key per lane) and once transposed
 // (the second, O^T = V^T P^T, reads 8 keys of a number per lane): the transposition happens on
 // the way into LDS, the cache keeps the rows only.  With many rows per sequence (a prompt) the
@@ -45,7 +48,7 @@ struct LatentLds {
     static constexpr int BYTES = (AL_KEYS * K_ROW + DT * 16 * AL_VROW + DT * 2 * 32) * 2;
 };
 
-template <int KD, int DT>
+template <int KD, int DT, int RT>
 __global__ void __launch_bounds__(256)
 attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, const bf16_t* __restrict__ cache,
                         const int* __restrict__ block_table, int bt_width, const int* __restrict__ cu_seqlens,
@@ -64,19 +67,15 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     for (; b < n_seqs; ++b) {
         tok0 = cu_seqlens[b];
         n_rows = (cu_seqlens[b + 1] - tok0) * n_heads;
-        int tiles = (n_rows + AL_ROWS - 1) / AL_ROWS;
+        int tiles = (n_rows + AL_ROWS * RT - 1) / (AL_ROWS * RT);
         if (tile < tiles) break;
         tile -= tiles;
     }
     if (b >= n_seqs) return;
     const int* pages = block_table + (size_t)b * bt_width;
     int pos0 = token_pos[tok0];
-    int row0 = tile * AL_ROWS, row1 = min(n_rows, row0 + AL_ROWS) - 1;        // the block's rows
-    int my_row = row0 + wave * 16 + col;
-    bool row_ok = my_row <= row1;
-    int my_pos = pos0 + (row_ok ? my_row : row1) / n_heads;
-    int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
-    int w_first = row0 + wave * 16, w_last = min(row1, w_first + 15);
+    int row0 = tile * AL_ROWS * RT, row1 = min(n_rows, row0 + AL_ROWS * RT) - 1;        // the block's rows
+    int w_first = row0 + wave * 16 * RT, w_last = min(row1, w_first + 16 * RT - 1);    // the wave's rows
     bool wave_active = w_first <= row1;
     int wave_lo = window > 0 ? max(0, pos0 + w_first / n_heads - window + 1) : 0;     // first key any of the wave's rows sees
     int wave_hi = pos0 + w_last / n_heads;                                            // last key
@@ -87,22 +86,32 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
     // zeros where the sizes stop short of the tiles: they are never written again
     for (int i = tid; i < L::BYTES / 16; i += 256) al_smem[i] = make_uint4(0u, 0u, 0u, 0u);
 
-    // Q^T operand: column = row of work, 8 numbers per lane and step
-    size_t grow = (size_t)tok0 * n_heads + (row_ok ? my_row : row1);
-    bf16x8_t qf[KD];
-    {
-        const bf16_t* qrow = q + grow * dk + g * 8;
+    // Per tile of 16 rows: the lane's column is one row of work.  Q^T operand: 8 numbers per lane and step.
+    bool row_ok[RT];
+    int my_pos[RT], my_lo[RT];
+    size_t grow[RT];
+    bf16x8_t qf[RT][KD];
+    float m[RT], l[RT];
+    f32x4_t o[RT][DT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        int my_row = w_first + rt * 16 + col;
+        row_ok[rt] = my_row <= row1;
+        my_pos[rt] = pos0 + (row_ok[rt] ? my_row : row1) / n_heads;
+        my_lo[rt] = window > 0 ? max(0, my_pos[rt] - window + 1) : 0;
+        grow[rt] = (size_t)tok0 * n_heads + (row_ok[rt] ? my_row : row1);
+        const bf16_t* qrow = q + grow[rt] * dk + g * 8;
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd) {
-            bool ok = row_ok && kd * 32 + g * 8 < dk;
+            bool ok = row_ok[rt] && kd * 32 + g * 8 < dk;
             uint4 v = ok ? *(const uint4*)(qrow + kd * 32) : make_uint4(0u, 0u, 0u, 0u);
-            qf[kd] = __builtin_bit_cast(bf16x8_t, v);
+            qf[rt][kd] = __builtin_bit_cast(bf16x8_t, v);
         }
-    }
-    float m = -INFINITY, l = 0.f;
-    f32x4_t o[DT];
+        m[rt] = -INFINITY;
+        l[rt] = 0.f;
 #pragma unroll
-    for (int i = 0; i < DT; ++i) o[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < DT; ++i) o[rt][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
 
     // A piece on its way: a thread takes the two keys of a column (see above) and 8 numbers of both.
     int dk8 = dk / 8, dv8 = dv / 8;
@@ -157,85 +166,98 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out, 
         int key0 = piece * AL_KEYS;
         if (!wave_active || key0 > wave_hi || key0 + AL_KEYS - 1 < wave_lo) continue;      // wave-uniform
         // scores of 2 x 16 keys: row r of tile u is key 8 (r / 4) + 4 u + r % 4, so that element i of
-        // s[u] in lane (g, col) is key 8 g + 4 u + i of the column's row of work
-        f32x4_t s[2];
+        // s[rt][u] in lane (g, col) is key 8 g + 4 u + i of the column's row of work
+        f32x4_t s[RT][2];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) s[rt][u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
             const bf16_t* krow = sk + (16 * u + col) * L::K_ROW + g * 8;       // key 8 (col / 4) + 4 u + col % 4
 #pragma unroll
             for (int kd = 0; kd < KD; ++kd) {
                 bf16x8_t kf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(krow + kd * 32));
-                s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kd], s[u], 0, 0, 0);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    s[rt][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[rt][kd], s[rt][u], 0, 0, 0);
             }
         }
-        float mx = -INFINITY;
+        bf16x8_t pf[RT];
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int rt = 0; rt < RT; ++rt) {
+            float mx = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                int key = key0 + g * 8 + u * 4 + i;
-                float v = (row_ok && key >= my_lo && key <= my_pos) ? s[u][i] * scale_log2e : -INFINITY;
-                s[u][i] = v;
-                mx = fmaxf(mx, v);
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    int key = key0 + g * 8 + u * 4 + i;
+                    float v = (row_ok[rt] && key >= my_lo[rt] && key <= my_pos[rt]) ? s[rt][u][i] * scale_log2e : -INFINITY;
+                    s[rt][u][i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            // The exponents' reference m follows a row's maximum only when that has grown by more than
+            // AL_LAZY_MAX: any reference gives the same quotient at the end, the probabilities stay below
+            // 2^AL_LAZY_MAX, and the sums and outputs so far are rescaled only for a row's first pieces
+            // instead of with every piece (the outputs are the bulk of a lane's registers).
+            if (__builtin_amdgcn_ballot_w64(mx > m[rt] + AL_LAZY_MAX)) {
+                float m_new = fmaxf(m[rt], mx);
+                float corr = fast_exp2(m[rt] - (m_new == -INFINITY ? 0.f : m_new));
+                l[rt] *= corr;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[rt][dt] = o[rt][dt] * corr;
+                m[rt] = m_new;
             }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        // The exponents' reference m follows a row's maximum only when that has grown by more than
-        // AL_LAZY_MAX: any reference gives the same quotient at the end, the probabilities stay below
-        // 2^AL_LAZY_MAX, and the sums and outputs so far are rescaled only for a row's first pieces
-        // instead of with every piece (the outputs are the bulk of a lane's registers).
-        if (__builtin_amdgcn_ballot_w64(mx > m + AL_LAZY_MAX)) {
-            float m_new = fmaxf(m, mx);
-            float corr = fast_exp2(m - (m_new == -INFINITY ? 0.f : m_new));
-            l *= corr;
+            float m_use = m[rt] == -INFINITY ? 0.f : m[rt];
+            float sum = 0.f;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o[dt] = o[dt] * corr;
-            m = m_new;
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    s[rt][u][i] = fast_exp2(s[rt][u][i] - m_use);
+                    sum += s[rt][u][i];
+                }
+            sum += __shfl_xor(sum, 16, 64);
+            sum += __shfl_xor(sum, 32, 64);
+            l[rt] += sum;
+            // P^T operand: slot 2 i + u = key 8 g + 4 u + i, the order of the transposed copy
+            pf[rt] = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(s[rt][0][0], s[rt][1][0]), pack_bf16x2(s[rt][0][1], s[rt][1][1]),
+                                                             pack_bf16x2(s[rt][0][2], s[rt][1][2]), pack_bf16x2(s[rt][0][3], s[rt][1][3])));
         }
-        float m_use = m == -INFINITY ? 0.f : m;
-        float sum = 0.f;
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                s[u][i] = fast_exp2(s[u][i] - m_use);
-                sum += s[u][i];
-            }
-        sum += __shfl_xor(sum, 16, 64);
-        sum += __shfl_xor(sum, 32, 64);
-        l += sum;
-        // P^T operand: slot 2 i + u = key 8 g + 4 u + i, the order of the transposed copy
-        bf16x8_t pf = __builtin_bit_cast(bf16x8_t, make_uint4(pack_bf16x2(s[0][0], s[1][0]), pack_bf16x2(s[0][1], s[1][1]),
-                                                              pack_bf16x2(s[0][2], s[1][2]), pack_bf16x2(s[0][3], s[1][3])));
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             bf16x8_t vf = __builtin_bit_cast(bf16x8_t, *(const uint4*)(sv + al_vrow_at(dt * 16 + col) + g * 8));
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[dt], 0, 0, 0);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                o[rt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[rt], o[rt][dt], 0, 0, 0);
         }
     }
-    if (!row_ok) return;
-    // element i of o[dt] is number 16 dt + 4 g + i of the column's row
-    if (n_splits == 1) {
-        float inv = 1.0f / l;
-        bf16_t* orow = out + grow * dv;
+    // element i of o[rt][dt] is number 16 dt + 4 g + i of the column's row
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            int d = dt * 16 + 4 * g;
-            if (d < dv)       // (dv is a multiple of 8: four numbers are inside or outside together)
-                *(uint2*)(orow + d) = make_uint2(pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv), pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv));
-        }
-    } else {
-        size_t slot = grow * n_splits + split;
-        float* po = part_o + slot * dv;
+    for (int rt = 0; rt < RT; ++rt) {
+        if (!row_ok[rt]) continue;
+        if (n_splits == 1) {
+            float inv = 1.0f / l[rt];
+            bf16_t* orow = out + grow[rt] * dv;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            int d = dt * 16 + 4 * g;
-            if (d < dv) *(float4*)(po + d) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
-        }
-        if (g == 0) {
-            part_ml[slot * 2] = m;
-            part_ml[slot * 2 + 1] = l;
+            for (int dt = 0; dt < DT; ++dt) {
+                int d = dt * 16 + 4 * g;
+                if (d < dv)       // (dv is a multiple of 8: four numbers are inside or outside together)
+                    *(uint2*)(orow + d) = make_uint2(pack_bf16x2(o[rt][dt][0] * inv, o[rt][dt][1] * inv),
+                                                     pack_bf16x2(o[rt][dt][2] * inv, o[rt][dt][3] * inv));
+            }
+        } else {
+            size_t slot = grow[rt] * n_splits + split;
+            float* po = part_o + slot * dv;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                int d = dt * 16 + 4 * g;
+                if (d < dv) *(float4*)(po + d) = make_float4(o[rt][dt][0], o[rt][dt][1], o[rt][dt][2], o[rt][dt][3]);
+            }
+            if (g == 0) {
+                part_ml[slot * 2] = m[rt];
+                part_ml[slot * 2 + 1] = l[rt];
+            }
         }
     }
 }
