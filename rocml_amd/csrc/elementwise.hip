@@ -426,7 +426,7 @@ qk_norm_rope_rows_kernel(
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     TO* __restrict__ q_out, TO* __restrict__ kcache, const int* __restrict__ block_table, int bt_width,
     const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size, int rows_per_token,
-    int first_row) {
+    int first_row, const float* __restrict__ bias) {
     constexpr int HJ = QK_PER_LANE / 2;
     int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
     long long total = (long long)n_tokens * rows_per_token;
@@ -441,6 +441,10 @@ qk_norm_rope_rows_kernel(
         const TI* src = qkv + (size_t)tok[i] * ld + (size_t)rr[i] * d;
 #pragma unroll
         for (int j = 0; j < QK_PER_LANE; ++j) v[i][j] = Elem<TI>::load(src + lane + j * WAVE);
+        if (bias) {
+#pragma unroll
+            for (int j = 0; j < QK_PER_LANE; ++j) v[i][j] += bias[(size_t)rr[i] * d + lane + j * WAVE];
+        }
         if (cos_t) {
 #pragma unroll
             for (int j = 0; j < HJ; ++j) {
@@ -561,7 +565,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     // (and the pairs are (e, e + d/2): neighbours as pairs go through LDS)
     bool local_pair = per_lane >= 2 && (rot == 0 || (rot == d && pairing == 0)) && d == per_lane * WAVE && dv == d;
     // many rows, none of them values: several rows per wave
-    bool many_rows = !bias && local_pair && per_lane <= 4 && n_splits == 1 && n_tokens >= VT_TOKENS && (v_tiled || !write_kv);
+    bool many_rows = local_pair && per_lane <= 4 && n_splits == 1 && n_tokens >= VT_TOKENS && (v_tiled || !write_kv);
     constexpr int MANY = 4;
     int grid = many_rows ? ceil_div(rows, QK_WAVES * MANY) : ceil_div(rows, QK_WAVES);
     size_t lds = local_pair ? 0 : (size_t)QK_WAVES * d * sizeof(float);
@@ -574,7 +578,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     qk_norm_rope_rows_kernel<TI, TO, N, MANY><<<grid, EW_BLOCK, 0, stream>>>(                   \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, rot ? cos_t : nullptr,   \
         rot ? sin_t : nullptr, (TO*)q_out, (TO*)kcache, block_table, bt_width, token_seq,       \
-        token_pos, page_size, rows_per_token, first_row)
+        token_pos, page_size, rows_per_token, first_row, bias)
 #define LAUNCH(TI, TO)                                                                          \
     {                                                                                           \
         if (many_rows) { if (per_lane == 2) LAUNCH_ROWS(TI, TO, 2); else LAUNCH_ROWS(TI, TO, 4); } \

@@ -231,11 +231,12 @@ def test_relu_gated_product(dtype, tol, m):
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)])
 @pytest.mark.parametrize("T", [3, 150])
-def test_biased_projection_rows_into_the_cache(dtype, tol, T):
+@pytest.mark.parametrize("D,DV", [(32, 80), (128, 128)])
+def test_biased_projection_rows_into_the_cache(dtype, tol, T, D, DV):
     """q and k rows get bias and per-head norm, v rows (of another size) their bias; k and v land in the pages."""
     from rocml_amd import ops
     gen = torch.Generator().manual_seed(T)
-    H, G, D, DV = 4, 2, 32, 80
+    H, G = 4, 2
     ld = (H + G) * D + G * DV
     qkv, bias = torch.randn(T, ld, generator=gen), torch.randn(ld, generator=gen)
     qg, kg = 1 + 0.3 * torch.randn(D, generator=gen), 1 + 0.3 * torch.randn(D, generator=gen)
