@@ -39,19 +39,17 @@ static int launch_decode_kernel(const AttnArgs& a, int n_splits, float* part_o, 
     int group = a.hq / a.hkv;
     int lds = WAVES * group * (D + 4) * (int)sizeof(float);
     dim3 grid(n_splits, a.hkv, a.n_tokens);
-    if constexpr (!FUSED) {
-        if (a.has_extra) {
-            static int allowed_extra = 0;
-            if (lds > allowed_extra) {
-                if (allow_lds(attn_decode_mfma_kernel<D, false, AHEAD, WAVES, true>, lds)) return 1;
-                allowed_extra = lds;
-            }
-            attn_decode_mfma_kernel<D, false, AHEAD, WAVES, true><<<grid, 64 * WAVES, lds, stream>>>(
-                a.q, a.out, const_cast<bf16_t*>(a.kcache), const_cast<bf16_t*>(a.vcache), a.block_table, a.bt_width,
-                a.token_seq, a.token_pos, a.hq, a.hkv, a.scale * LOG2E, a.window, n_splits, part_o, part_ml,
-                DecodeProj{}, a.extra);
-            return 0;
+    if (a.has_extra) {
+        static int allowed_extra = 0;
+        if (lds > allowed_extra) {
+            if (allow_lds(attn_decode_mfma_kernel<D, FUSED, AHEAD, WAVES, true>, lds)) return 1;
+            allowed_extra = lds;
         }
+        attn_decode_mfma_kernel<D, FUSED, AHEAD, WAVES, true><<<grid, 64 * WAVES, lds, stream>>>(
+            a.q, a.out, const_cast<bf16_t*>(a.kcache), const_cast<bf16_t*>(a.vcache), a.block_table, a.bt_width,
+            a.token_seq, a.token_pos, a.hq, a.hkv, a.scale * LOG2E, a.window, n_splits, part_o, part_ml,
+            FUSED ? *a.proj : DecodeProj{}, a.extra);
+        return 0;
     }
     static int allowed = 0;
     if (lds > allowed) {
@@ -306,7 +304,10 @@ ROCML_EXPORT int rocml_attention_decode_fused(const float* qkv, int ld, int qkv_
                                               int hkv, int d, int page_size, float scale, int window,
                                               int max_len, int n_splits, void* workspace,
                                               long long workspace_bytes, const float* row_ssq, int row_parts,
-                                              float row_eps, int row_width, hipStream_t stream) {
+                                              float row_eps, int row_width, const float* bias, int chunk,
+                                              const float* slopes, int sink, hipStream_t stream) {
+    // bias (may be null): [ld] numbers added to the projection's sums; chunk, slopes, sink: see MaskExtra.
+    ROCML_REQUIRE(chunk >= 0 && (chunk == 0 || window == 0), "fused decode attention: a window or blocks of positions, not both");
     ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && bt_width > 0 && qkv_splits >= 1,
                   "fused decode attention: bad sizes T=%d Hq=%d Hkv=%d width=%d splits=%d", n_tokens, hq, hkv,
                   bt_width, qkv_splits);
@@ -327,10 +328,12 @@ ROCML_EXPORT int rocml_attention_decode_fused(const float* qkv, int ld, int qkv_
     ROCML_REQUIRE(!row_ssq || (row_parts > 0 && row_eps > 0.f && row_width > 0),
                   "fused decode attention: a row scale needs parts, eps and the norm's width");
     DecodeProj pj{qkv, ld, qkv_splits, qkv_split_stride, q_gain, k_gain, eps, cos_t, sin_t, write_kv,
-                  row_ssq, row_parts, row_eps, row_ssq ? 1.0f / (float)row_width : 0.f};
+                  row_ssq, row_parts, row_eps, row_ssq ? 1.0f / (float)row_width : 0.f, bias};
     AttnArgs a{nullptr, (bf16_t*)out, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, bt_width,
                token_seq, token_pos, nullptr, 0, n_tokens, 0, max_len, hq, hkv, scale, window, workspace,
                workspace_bytes, n_splits, &pj};
+    a.extra = MaskExtra{chunk, slopes, sink};
+    a.has_extra = chunk > 0 || slopes || sink || bias;        // (the bias rides in the same instantiation)
     int rc = d == 64 ? launch_decode_fused<64>(a, stream)
              : d == 128 ? launch_decode_fused<128>(a, stream)
              : d == 192 ? launch_decode_fused<192>(a, stream) : launch_decode_fused<256>(a, stream);

@@ -52,6 +52,8 @@ struct DecodeProj {
     const float* q_gain; const float* k_gain; float eps;
     const float* cos_t; const float* sin_t; int write_kv;
     const float* row_ssq; int row_parts; float row_eps; float row_inv_width;
+    const float* bias;      // null: none; else one number per column of a projection row, added to the sums
+                            // (behind the row scale: the bias is no part of the normed input's product)
 };
 
 // grid (n_splits, Hkv, tokens), 4 or 8 waves; the block's pages are cut into 32-key pieces that the
@@ -83,7 +85,6 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                         int hkv, float scale_log2e, int window, int n_splits,
                         float* __restrict__ part_o, float* __restrict__ part_ml, DecodeProj pj,
                         MaskExtra mx = MaskExtra{}) {
-    static_assert(!(FUSED && EXTRA), "the kernel that reads the projection knows plain layers only");
     constexpr int KD = D / 32;      // MFMA steps along D for the scores
     constexpr int DT = D / 16;      // 16-row tiles of the output
     constexpr int THREADS = 64 * WAVES;
@@ -193,14 +194,14 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
             row_scale = 1.0f / sqrtf(wave_sum(ss) * pj.row_inv_width + pj.row_eps);
         }
         for (int base = 0; base < n_rows; base += 2 * WAVES) {
-            int r[2];
+            int r[2], prow[2];
             const float* src[2];
             float raw[2][J][4];
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
                 r[i] = base + i * WAVES + wave;
-                int prow = r[i] < group ? kvh * group + r[i] : (r[i] == group ? hq + kvh : hq + hkv + kvh);
-                src[i] = tok + (size_t)(r[i] < n_rows ? prow : 0) * D + lane;
+                prow[i] = r[i] < group ? kvh * group + r[i] : (r[i] == group ? hq + kvh : hq + hkv + kvh);
+                src[i] = tok + (size_t)(r[i] < n_rows ? prow[i] : 0) * D + lane;
 #pragma unroll
                 for (int j = 0; j < J; ++j)
 #pragma unroll
@@ -219,6 +220,9 @@ attn_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                         if (sp < pj.n_splits) a += raw[i][j][sp];
                     for (int sp = 4; sp < pj.n_splits; ++sp) a += src[i][j * 64 + sp * pj.split_stride];
                     val[i][j] = a * row_scale;
+                    if constexpr (EXTRA) {
+                        if (pj.bias && r[i] < n_rows) val[i][j] += pj.bias[(size_t)prow[i] * D + lane + j * 64];
+                    }
                 }
                 const float* gain = r[i] < group ? pj.q_gain : (r[i] == group ? pj.k_gain : nullptr);
                 if (gain) {

@@ -50,7 +50,7 @@ _SIGNATURES = {
         "rocml_attention": [_P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _I,
                             _P, _I, _I, _P, _I, _I, _P, _LL, _I, _I, _I, _P, _I, _P],
         "rocml_attention_decode_fused": [_P, _I, _I, _LL, _P, _P, _F, _P, _P, _I, _P, _P, _P, _P, _I, _P, _P,
-                                         _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P, _I, _F, _I, _P],
+                                         _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _LL, _P, _I, _F, _I, _P, _I, _P, _I, _P],
         "rocml_attention_prefill_fused": [_P, _I, _P, _F, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I,
                                           _P, _I, _P, _P],
     },
@@ -699,14 +699,26 @@ def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.
                            q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
                            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], write_kv: bool = True,
                            window: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
-                           max_len: int = 0, n_splits: int = 0, row_scale: Optional[RowScale] = None) -> None:
+                           max_len: int = 0, n_splits: int = 0, row_scale: Optional[RowScale] = None,
+                           bias: Optional[torch.Tensor] = None, chunk: Optional[int] = None,
+                           slopes: Optional[torch.Tensor] = None, sink: bool = False) -> None:
     """A decode step's attention straight from the q/k/v projection ``qkv`` (float32
     ``[tokens, ld]``, or its split-K partial sums ``[splits, tokens, ld]``): per-head norm,
     rotation, append of the new key and value to the cache and attention over the cache in one
     launch.  ``token_seq`` None: token ``t`` is the one token of the step's sequence ``t`` (row
     ``t`` of the block table).  ``workspace`` must not overlap ``qkv``.  ``row_scale``: the
-    projection's operand lacked its norm's scale, which is applied to the projection's sums here."""
-    _dev(qkv, out, k_cache, v_cache, block_table, token_seq, token_pos, q_gain, k_gain, cos, sin)
+    projection's operand lacked its norm's scale, which is applied to the projection's sums here.
+    ``bias`` (32-bit, one number per column of a projection row) is added behind that scale;
+    ``chunk``, ``slopes`` and ``sink`` as in ``attention``."""
+    _dev(qkv, out, k_cache, v_cache, block_table, token_seq, token_pos, q_gain, k_gain, cos, sin, bias, slopes)
+    if bias is not None:
+        _want(bias, torch.float32, "projection bias")
+        if bias.numel() < (n_heads + 2 * n_kv_heads) * head_dim and (write_kv or bias.numel() < n_heads * head_dim):
+            raise KernelError("the bias is shorter than a projection row")
+    if slopes is not None:
+        _want(slopes, torch.float32, "distance slopes")
+        if slopes.numel() != n_heads:
+            raise KernelError("one distance slope per query head is needed")
     _want(qkv, torch.float32, "projection output")
     qkv_splits, split_stride = 1, 0
     if qkv.dim() == 3:
@@ -751,7 +763,7 @@ def attention_decode_fused(qkv: torch.Tensor, out: torch.Tensor, k_cache: torch.
         1 if write_kv else 0, _ptr(out), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1],
         _ptr(token_seq), _ptr(token_pos), n_tokens, n_heads, n_kv_heads, head_dim, page, scale,
         0 if window is None else int(window), max_len, n_splits, ws_ptr, ws_bytes, ssq_ptr, parts, row_eps, width,
-        _stream()))
+        _ptr(bias), 0 if chunk is None else int(chunk), _ptr(slopes), 1 if sink else 0, _stream()))
 
 
 # ---- sampling ------------------------------------------------------------------------

@@ -125,7 +125,8 @@ class Attention(Mixer):
 
     def _fused_decode(self, step) -> bool:
         rot = None if self.position is None else self.position.rot_dim
-        return not self.extras and not self.spec.bias and step.max_new == 1 and ops.attention_decode_fusable(
+        # (blocks, slopes, a sink and biases ride in the fused kernel; a value head of another size does not)
+        return self.v_head_dim == self.spec.head_dim and step.max_new == 1 and ops.attention_decode_fusable(
             self.dtype, self.spec.n_heads, self.spec.n_kv_heads, self.spec.head_dim, ops.FUSED_DECODE_PAGE, rot, self.pairing)
 
     def _fused_prefill(self, step, cache) -> bool:
@@ -184,7 +185,9 @@ class Attention(Mixer):
                                        s.n_heads, s.n_kv_heads, s.head_dim, s.scale, self.q_gain, self.k_gain, eps,
                                        cos, sin, write_kv=owns_cache, window=s.window, workspace=scratch[used:],
                                        max_len=step.max_len, n_splits=self._decode_splits(step, cache),
-                                       row_scale=stream(step).row_scale)
+                                       row_scale=stream(step).row_scale,
+                                       bias=None if self.b_qkv is None else self.b_qkv[:rows], chunk=s.chunk,
+                                       slopes=self.slopes, sink=s.sink)
         else:
             if stream(step).row_scale is not None:
                 raise ConfigError("the attention was handed an input without its norm's scale in a step it cannot scale")
