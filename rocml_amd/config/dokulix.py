@@ -227,5 +227,8 @@ def checkpoint_names(spec: ModelSpec) -> Dict[str, str]:
 
 def unused_tensors(spec: ModelSpec) -> Tuple[str, ...]:
     """Tensors a checkpoint may hold that the model does not read: the second norm of a layer
-    without a feed-forward."""
-    return tuple(f"l{i}.norm2" for i, block in enumerate(spec.layers) if block.ffn is None)
+    without a feed-forward, the loop's vectors of a model without a loop."""
+    names = [f"l{i}.norm2" for i, block in enumerate(spec.layers) if block.ffn is None]
+    if not spec.pass_offsets:
+        names.append("loop.step")
+    return tuple(names)
