@@ -537,7 +537,7 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     long long split_stride, const float* bias, int dv, hipStream_t stream) {
     // bias (may be null): [ld] numbers added to the projection's sums; dv (0: d): value head size.
     if (dv <= 0) dv = d;
-    ROCML_REQUIRE(n_tokens >= 0 && hq > 0 && hkv > 0 && d > 0, "qk_norm_rope_append: bad sizes");
+    ROCML_REQUIRE(n_tokens >= 0 && (hq > 0 || (hq == 0 && !q_out)) && hkv > 0 && d > 0, "qk_norm_rope_append: bad sizes");
     ROCML_REQUIRE(dv <= QK_MAX_PER_LANE * WAVE, "qk_norm_rope_append: value head size %d exceeds %d", dv,
                   QK_MAX_PER_LANE * WAVE);
     ROCML_REQUIRE(n_splits >= 1 && (n_splits == 1 || (split_stride > 0 && in_dtype == ROCML_F32)),
@@ -730,18 +730,24 @@ ROCML_EXPORT int rocml_latent_prepare(const float* proj, int ld, int n_tokens, i
 // The rotated part of every query head: q [T, ldq] holds, per head, head_stride numbers of which
 // those from `offset` on, rot_part of them, are the part; its rotation (as above) goes to
 // out [T, ldo] at out_offset of each head's out_stride numbers.
+// lead: so many numbers before the part are copied unchanged in front of it (out_offset is where they start).
 template <typename TO>
 __global__ void rope_heads_kernel(const float* __restrict__ q, int ldq, int head_stride, int offset, int rot_part,
                                   int dims, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                   TO* __restrict__ out, int ldo, int out_stride, int out_offset, int n_heads,
-                                  long long total) {
+                                  int lead, long long total) {
     long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
     if (idx >= total) return;
-    int e = (int)(idx % rot_part);
-    long long th = idx / rot_part;
+    int width = lead + rot_part;
+    int e = (int)(idx % width) - lead;
+    long long th = idx / width;
     int h = (int)(th % n_heads);
     long long t = th / n_heads;
     const float* src = q + (size_t)t * ldq + (size_t)h * head_stride + offset;
+    if (e < 0) {
+        Elem<TO>::store(out + (size_t)t * ldo + (size_t)h * out_stride + out_offset + lead + e, src[e]);
+        return;
+    }
     int half = dims / 2;
     float v = src[e];
     if (e < half) {
@@ -749,27 +755,28 @@ __global__ void rope_heads_kernel(const float* __restrict__ q, int ldq, int head
     } else if (e < dims) {
         v = src[e] * cos_t[t * half + e - half] + src[e - half] * sin_t[t * half + e - half];
     }
-    Elem<TO>::store(out + (size_t)t * ldo + (size_t)h * out_stride + out_offset + e, v);
+    Elem<TO>::store(out + (size_t)t * ldo + (size_t)h * out_stride + out_offset + lead + e, v);
 }
 
 ROCML_EXPORT int rocml_rope_heads(const float* q, int ldq, int head_stride, int offset, int rot_part, int dims,
                                   const float* cos_t, const float* sin_t, void* out, int out_dtype, int ldo,
-                                  int out_stride, int out_offset, int n_tokens, int n_heads, hipStream_t stream) {
+                                  int out_stride, int out_offset, int n_tokens, int n_heads, int lead,
+                                  hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && n_heads > 0 && rot_part >= 0 && dims >= 0 && dims % 2 == 0 && dims <= rot_part,
                   "rope_heads: bad sizes T=%d H=%d part=%d dims=%d", n_tokens, n_heads, rot_part, dims);
-    ROCML_REQUIRE(offset >= 0 && offset + rot_part <= head_stride && ldq >= n_heads * head_stride &&
-                      out_offset >= 0 && out_offset + rot_part <= out_stride && ldo >= n_heads * out_stride,
-                  "rope_heads: the part does not lie inside the heads");
+    ROCML_REQUIRE(lead >= 0 && offset >= lead && offset + rot_part <= head_stride && ldq >= n_heads * head_stride &&
+                      out_offset >= 0 && out_offset + lead + rot_part <= out_stride && ldo >= n_heads * out_stride,
+                  "rope_heads: the part (and what is copied before it) does not lie inside the heads");
     ROCML_REQUIRE(dims == 0 || (cos_t && sin_t), "rope_heads: rotation tables missing");
-    long long total = (long long)n_tokens * n_heads * rot_part;
+    long long total = (long long)n_tokens * n_heads * (lead + rot_part);
     if (total == 0) return 0;
     int grid = ceil_div(total, EW_BLOCK);
     if (out_dtype == ROCML_F32)
         rope_heads_kernel<float><<<grid, EW_BLOCK, 0, stream>>>(q, ldq, head_stride, offset, rot_part, dims, cos_t, sin_t,
-                                                                (float*)out, ldo, out_stride, out_offset, n_heads, total);
+                                                                (float*)out, ldo, out_stride, out_offset, n_heads, lead, total);
     else if (out_dtype == ROCML_BF16)
         rope_heads_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>(q, ldq, head_stride, offset, rot_part, dims, cos_t, sin_t,
-                                                                 (bf16_t*)out, ldo, out_stride, out_offset, n_heads, total);
+                                                                 (bf16_t*)out, ldo, out_stride, out_offset, n_heads, lead, total);
     else return rocml_fail("rope_heads: unknown dtype code %d", out_dtype);
     ROCML_CHECK_LAUNCH("rope_heads");
     return 0;
@@ -795,5 +802,131 @@ ROCML_EXPORT int rocml_sigmoid_gate(void* y, int dtype, const float* g, int ldg,
     else if (dtype == ROCML_BF16) sigmoid_gate_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>((bf16_t*)y, g, ldg, n, total);
     else return rocml_fail("sigmoid_gate: unknown dtype code %d", dtype);
     ROCML_CHECK_LAUNCH("sigmoid_gate");
+    return 0;
+}
+
+// ---- latent attention, prompts: the rows a step's queries can see, as a dense matrix ---------
+// A prompt step may expand keys and values per head for the positions its queries see (the step's own
+// tokens and up to window - 1 cached ones per sequence) and run the attention kernels for separate
+// heads over them.  The positions of sequence b are [lo_b, end_b), lo_b = max(0, start_b - window + 1)
+// (0 without a window); they lie in the sequence's pages fp_b .. lp_b, which get scratch pages
+// base_b .. in sequence order.  latent_window_plan (one block) writes the scratch block table
+// [n_seqs, width] (page index of the sequence -> scratch page, -1 elsewhere) and, per scratch page, the
+// latent pool page it mirrors, its first position and the range of positions that count; latent_window_gather
+// copies the rows (zeros where a position does not count) into rows [scratch page * 64 + place].
+__global__ void latent_window_plan_kernel(const int* __restrict__ cu_seqlens, const int* __restrict__ token_pos,
+                                          const int* __restrict__ block_table, int bt_width, int n_seqs, int window,
+                                          int page_size, int* __restrict__ table, int width, int* __restrict__ src_page,
+                                          int* __restrict__ first_pos, int* __restrict__ lo_pos, int* __restrict__ hi_pos,
+                                          int max_pages) {
+    extern __shared__ int plan_smem[];      // [n_seqs] base, [n_seqs] first page, [n_seqs] count
+    int* base = plan_smem;
+    int* fpage = plan_smem + n_seqs;
+    int* count = plan_smem + 2 * n_seqs;
+    if (threadIdx.x == 0) {
+        int at = 0;
+        for (int b = 0; b < n_seqs; ++b) {
+            int start = token_pos[cu_seqlens[b]], end = start + cu_seqlens[b + 1] - cu_seqlens[b];
+            int lo = window > 0 ? max(0, start - window + 1) : 0;
+            fpage[b] = lo / page_size;
+            count[b] = (end - 1) / page_size - fpage[b] + 1;
+            base[b] = at;
+            at += count[b];
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < max_pages; i += blockDim.x) src_page[i] = -1;
+    for (int i = threadIdx.x; i < n_seqs * width; i += blockDim.x) table[i] = -1;
+    __syncthreads();
+    for (int b = 0; b < n_seqs; ++b) {
+        int start = token_pos[cu_seqlens[b]], end = start + cu_seqlens[b + 1] - cu_seqlens[b];
+        int lo = window > 0 ? max(0, start - window + 1) : 0;
+        for (int i = threadIdx.x; i < count[b]; i += blockDim.x) {
+            int p = fpage[b] + i, s = base[b] + i;
+            if (s >= max_pages || p >= width || p >= bt_width) continue;
+            table[(size_t)b * width + p] = s;
+            src_page[s] = block_table[(size_t)b * bt_width + p];
+            first_pos[s] = p * page_size;
+            lo_pos[s] = lo;
+            hi_pos[s] = end;
+        }
+    }
+}
+
+template <typename T>
+__global__ void latent_window_gather_kernel(const T* __restrict__ cache, int row, int page_size,
+                                            const int* __restrict__ src_page, const int* __restrict__ first_pos,
+                                            const int* __restrict__ lo_pos, const int* __restrict__ hi_pos,
+                                            T* __restrict__ out, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    int e = (int)(idx % row);
+    long long r = idx / row;
+    int s = (int)(r / page_size), i = (int)(r % page_size);
+    int page = src_page[s];
+    T v = 0;
+    if (page >= 0) {
+        int pos = first_pos[s] + i;
+        if (pos >= lo_pos[s] && pos < hi_pos[s]) v = cache[((size_t)page * page_size + i) * row + e];
+    }
+    out[idx] = v;
+}
+
+ROCML_EXPORT int rocml_latent_window_plan(const int* cu_seqlens, const int* token_pos, const int* block_table, int bt_width,
+                                          int n_seqs, int window, int page_size, int* table, int width, int* plan,
+                                          int max_pages, hipStream_t stream) {
+    // plan: 4 * max_pages ints (source page, first position, first and one past the last position that count)
+    ROCML_REQUIRE(n_seqs > 0 && n_seqs <= 4096 && bt_width > 0 && width > 0 && max_pages > 0 && page_size > 0 && window >= 0,
+                  "latent_window_plan: bad sizes sequences=%d width=%d pages=%d", n_seqs, width, max_pages);
+    latent_window_plan_kernel<<<1, 256, 3 * n_seqs * sizeof(int), stream>>>(
+        cu_seqlens, token_pos, block_table, bt_width, n_seqs, window, page_size, table, width, plan, plan + max_pages,
+        plan + 2 * max_pages, plan + 3 * max_pages, max_pages);
+    ROCML_CHECK_LAUNCH("latent_window_plan");
+    return 0;
+}
+
+ROCML_EXPORT int rocml_latent_window_gather(const void* cache, int dtype, int row, int page_size, const int* plan,
+                                            int max_pages, void* out, hipStream_t stream) {
+    ROCML_REQUIRE(row > 0 && page_size > 0 && max_pages > 0, "latent_window_gather: bad sizes");
+    long long total = (long long)max_pages * page_size * row;
+    int grid = ceil_div(total, EW_BLOCK);
+    if (dtype == ROCML_BF16)
+        latent_window_gather_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)cache, row, page_size, plan,
+            plan + max_pages, plan + 2 * max_pages, plan + 3 * max_pages, (bf16_t*)out, total);
+    else if (dtype == ROCML_F32)
+        latent_window_gather_kernel<float><<<grid, EW_BLOCK, 0, stream>>>((const float*)cache, row, page_size, plan,
+            plan + max_pages, plan + 2 * max_pages, plan + 3 * max_pages, (float*)out, total);
+    else return rocml_fail("latent_window_gather: unknown dtype code %d", dtype);
+    ROCML_CHECK_LAUNCH("latent_window_gather");
+    return 0;
+}
+
+// out[t, h * n + i] = x[t, h * x_stride + i] * sigmoid(g[t, h * n + i]) (g null: a plain copy of the heads'
+// leading n numbers): the heads of an attention output that is wider than the values, gated and packed.
+template <typename T>
+__global__ void gate_heads_kernel(const T* __restrict__ x, int ldx, int x_stride, const float* __restrict__ g, int ldg,
+                                  T* __restrict__ out, int n_heads, int n, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    int i = (int)(idx % n);
+    long long th = idx / n;
+    int h = (int)(th % n_heads);
+    long long t = th / n_heads;
+    float v = Elem<T>::load(x + (size_t)t * ldx + (size_t)h * x_stride + i);
+    if (g) v *= 1.0f / (1.0f + expf(-g[(size_t)t * ldg + (size_t)h * n + i]));
+    Elem<T>::store(out + idx, v);
+}
+
+ROCML_EXPORT int rocml_gate_heads(const void* x, int dtype, int ldx, int x_stride, const float* g, int ldg, void* out,
+                                  int n_rows, int n_heads, int n, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && n_heads > 0 && n > 0 && n <= x_stride && ldx >= n_heads * x_stride && (!g || ldg >= n_heads * n),
+                  "gate_heads: bad sizes rows=%d heads=%d n=%d stride=%d", n_rows, n_heads, n, x_stride);
+    long long total = (long long)n_rows * n_heads * n;
+    if (total == 0) return 0;
+    int grid = ceil_div(total, EW_BLOCK);
+    if (dtype == ROCML_F32) gate_heads_kernel<float><<<grid, EW_BLOCK, 0, stream>>>((const float*)x, ldx, x_stride, g, ldg, (float*)out, n_heads, n, total);
+    else if (dtype == ROCML_BF16) gate_heads_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)x, ldx, x_stride, g, ldg, (bf16_t*)out, n_heads, n, total);
+    else return rocml_fail("gate_heads: unknown dtype code %d", dtype);
+    ROCML_CHECK_LAUNCH("gate_heads");
     return 0;
 }

@@ -36,7 +36,10 @@ _SIGNATURES = {
         "rocml_add_into": [_P, _P, _I, _LL, _P],
         "rocml_add_row_vector": [_P, _P, _I, _I, _P],
         "rocml_latent_prepare": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _P],
-        "rocml_rope_heads": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+        "rocml_rope_heads": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+        "rocml_latent_window_plan": [_P, _P, _P, _I, _I, _I, _I, _P, _I, _P, _I, _P],
+        "rocml_latent_window_gather": [_P, _I, _I, _I, _P, _I, _P, _P],
+        "rocml_gate_heads": [_P, _I, _I, _I, _P, _I, _P, _I, _I, _I, _P],
         "rocml_sigmoid_gate": [_P, _I, _P, _I, _I, _I, _P],
     },
     "gemm": {
@@ -342,10 +345,11 @@ def latent_prepare(proj: torch.Tensor, q_rank: int, kv_rank: int, rot_part: int,
 
 def rope_heads(q: torch.Tensor, n_heads: int, head_stride: int, offset: int, rot_part: int, rot_dims: int,
                cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], out: torch.Tensor, out_stride: int,
-               out_offset: int) -> None:
+               out_offset: int, lead: int = 0) -> None:
     """The part of every head of ``q [T, n_heads * head_stride]`` (32-bit) that starts at ``offset``
     and is ``rot_part`` wide, rotated (its first ``rot_dims`` numbers, pairs ``(i, i + rot_dims/2)``),
-    written to ``out [T, n_heads * out_stride]`` at ``out_offset`` of every head."""
+    written to ``out [T, n_heads * out_stride]`` at ``out_offset`` of every head.  ``lead``: so many
+    numbers before the part are copied unchanged in front of it (``out_offset`` is where they start)."""
     _dev(q, cos, sin, out)
     _want(q, torch.float32, "queries")
     n_tokens = q.shape[0]
@@ -356,7 +360,52 @@ def rope_heads(q: torch.Tensor, n_heads: int, head_stride: int, offset: int, rot
         raise KernelError(f"rotation tables must be float32 {(n_tokens, rot_dims // 2)}")
     _check("elementwise", library("elementwise").rocml_rope_heads(
         _ptr(q), q.shape[1], head_stride, offset, rot_part, rot_dims, _ptr(cos), _ptr(sin), _ptr(out), _code(out),
-        out.shape[1], out_stride, out_offset, n_tokens, n_heads, _stream()))
+        out.shape[1], out_stride, out_offset, n_tokens, n_heads, int(lead), _stream()))
+
+
+def latent_window_plan(cu_seqlens: torch.Tensor, token_pos: torch.Tensor, block_table: torch.Tensor, window: Optional[int],
+                       page_size: int, table: torch.Tensor, plan: torch.Tensor) -> None:
+    """For a prompt step over a cache of rows per position: which pages hold the positions the step's
+    queries see (per sequence its new tokens and up to ``window - 1`` before them; all without a
+    window), numbered as scratch pages in sequence order.  Writes ``table [sequences, width]``
+    (a sequence's page index -> scratch page, -1 elsewhere) and ``plan [4, max_pages]`` int32: per
+    scratch page the pool page it mirrors (-1: unused), its first position, and the first and one past
+    the last position that count."""
+    _dev(cu_seqlens, token_pos, block_table, table, plan)
+    for t, name in ((cu_seqlens, "sequence offsets"), (token_pos, "token positions"), (block_table, "block table"),
+                    (table, "scratch table"), (plan, "plan")):
+        _want(t, torch.int32, name)
+    n_seqs = cu_seqlens.numel() - 1
+    if table.dim() != 2 or table.shape[0] != n_seqs or plan.dim() != 2 or plan.shape[0] != 4 or block_table.shape[0] < n_seqs:
+        raise KernelError("the scratch table must be [sequences, width] and the plan [4, pages]")
+    _check("elementwise", library("elementwise").rocml_latent_window_plan(
+        _ptr(cu_seqlens), _ptr(token_pos), _ptr(block_table), block_table.shape[1], n_seqs, 0 if window is None else int(window),
+        page_size, _ptr(table), table.shape[1], _ptr(plan), plan.shape[1], _stream()))
+
+
+def latent_window_gather(cache: torch.Tensor, plan: torch.Tensor, out: torch.Tensor) -> None:
+    """The rows ``latent_window_plan`` planned, ``cache [pages, page_size, row]`` -> ``out [max_pages *
+    page_size, row]`` in scratch-page order, zeros where a position does not count."""
+    _dev(cache, plan, out)
+    _want(plan, torch.int32, "plan")
+    pages, page_size, row = cache.shape
+    if out.dtype != cache.dtype or out.shape != (plan.shape[1] * page_size, row):
+        raise KernelError(f"gathered rows must be {(plan.shape[1] * page_size, row)} of the cache's type")
+    _check("elementwise", library("elementwise").rocml_latent_window_gather(
+        _ptr(cache), _code(cache), row, page_size, _ptr(plan), plan.shape[1], _ptr(out), _stream()))
+
+
+def gate_heads(x: torch.Tensor, x_stride: int, gate: Optional[torch.Tensor], out: torch.Tensor, n_heads: int, n: int) -> None:
+    """``out[t, h * n + i] = x[t, h * x_stride + i] * sigmoid(gate[t, h * n + i])`` (``gate`` None: the
+    plain copy): the leading ``n`` numbers of every head of ``x``, gated and packed."""
+    _dev(x, out)
+    if gate is not None and (not gate.is_cuda or gate.dtype != torch.float32 or gate.stride(1) != 1 or gate.shape != out.shape):
+        raise KernelError("the gate must be 32-bit and of the output's shape")
+    if x.dtype != out.dtype or out.shape != (x.shape[0], n_heads * n) or x.shape[1] < n_heads * x_stride:
+        raise KernelError("gate_heads: shapes do not fit")
+    ldg = 0 if gate is None else (gate.stride(0) if x.shape[0] > 1 else max(gate.stride(0), gate.shape[1]))
+    _check("elementwise", library("elementwise").rocml_gate_heads(
+        _ptr(x), _code(x), x.shape[1], x_stride, _ptr(gate), ldg, _ptr(out), x.shape[0], n_heads, n, _stream()))
 
 
 def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> None:

@@ -36,6 +36,10 @@ from .residual import stream
 
 class LatentAttention(Mixer):
     adds_only = True
+    # A prompt step of at least so many tokens expands keys and values per head for the positions its
+    # queries see and runs the attention kernels for separate heads: a (query, key) pair then costs
+    # 2 (head_dim + rot_dim) + 2 v_head_dim operations instead of 2 (kv_rank + rot_dim) + 2 kv_rank.
+    EXPANDED_PROMPT_MIN_TOKENS = 256
 
     def __init__(self, spec: LatentAttentionSpec, ctx: BuildContext):
         for norm in (spec.q_norm, spec.kv_norm):
@@ -67,6 +71,8 @@ class LatentAttention(Mixer):
         self.w_o: Optional[torch.Tensor] = None
         self.q_gain: Optional[torch.Tensor] = None
         self.kv_gain: Optional[torch.Tensor] = None
+        self.w_expand: Optional[torch.Tensor] = None
+        self._ident = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         s = self.spec
@@ -93,6 +99,25 @@ class LatentAttention(Mixer):
         self.w_o = tensors["o_proj.weight"]
         self.q_gain = tensors["dq_norm.weight"]
         self.kv_gain = tensors["dkv_norm.weight"]
+        if self._expandable():
+            # One matrix that turns a cache row [c, k_r] into every head's key [W_uk,a c, k_r] and value
+            # [W_uv,a c, zeros up to the key's size]: rows of W_uk and W_uv against c, an identity against k_r.
+            D, H = self.qk_dim, s.n_heads
+            w = torch.zeros((2 * H, D, self.row), dtype=self.dtype, device=self.w_o.device)
+            w[:H, :s.head_dim, :s.kv_rank] = tensors["uk.weight"].view(H, s.head_dim, s.kv_rank)
+            w[:H, s.head_dim:, s.kv_rank:] = torch.eye(s.rot_dim, dtype=self.dtype, device=w.device)
+            w[H:, :s.v_head_dim, :s.kv_rank] = tensors["uv.weight"].view(H, s.v_head_dim, s.kv_rank)
+            self.w_expand = w.view(2 * H * D, self.row).contiguous()
+
+    def _expandable(self) -> bool:
+        """Whether prompts may take the expanded form: bfloat16, a head (unrotated and rotated part) of a
+        size the matrix-core attention kernels know, values no wider than that."""
+        return (self.dtype == torch.bfloat16 and self.qk_dim in ops.PREFILL_FUSED_HEAD_DIMS
+                and self.spec.v_head_dim <= self.qk_dim and self.row % 8 == 0)
+
+    def matrix_elements(self) -> int:
+        # (the expansion matrix is built from uk and uv: no parameters of its own)
+        return super().matrix_elements()
 
     def flops(self, new_counts, starts) -> int:
         s = self.spec
@@ -107,9 +132,15 @@ class LatentAttention(Mixer):
     def activation_bytes(self, n_tokens: int) -> int:
         s = self.spec
         size = 2 if self.dtype == torch.bfloat16 else 4
-        return n_tokens * ((self.first_cols + s.n_heads * self.qk_dim) * 4
-                           + (s.q_rank + s.n_heads * (self.row + s.kv_rank) + self.o_dim) * size
-                           + self.position.rot_dim * 4)
+        total = n_tokens * ((self.first_cols + s.n_heads * self.qk_dim) * 4
+                            + (s.q_rank + s.n_heads * (self.row + s.kv_rank) + self.o_dim) * size
+                            + self.position.rot_dim * 4)
+        if self._expandable():
+            # a prompt step's expanded keys and values (the step's tokens and a window before each sequence),
+            # as the product leaves them and as pages, and the queries and outputs of separate heads
+            keys = 2 * n_tokens + (s.window or 0)
+            total += keys * (self.row + 4 * s.n_heads * self.qk_dim) * size + 2 * n_tokens * s.n_heads * self.qk_dim * size
+        return total
 
     def cache_request(self) -> LatentCacheRequest:
         return LatentCacheRequest(self.row, self.spec.window)
@@ -132,6 +163,11 @@ class LatentAttention(Mixer):
         ops.gemm(cq, self.w_uq, q, workspace=ws.scratch())
         # the queries as the attention takes them: per head [W_uk^T q^n, rotated q^r]
         qa = ws.get("latent.qa", (n, s.n_heads * self.row), self.dtype)
+        expanded = (self.w_expand is not None and step.max_new > 1 and n >= self.EXPANDED_PROMPT_MIN_TOKENS
+                    and step.cu_seqlens is not None and cache.k.shape[1] == ops.PREFILL_FUSED_PAGE)
+        if expanded:
+            self._expanded_prompt(step, q, first, cos, sin, dims, cache, x_accum)
+            return
         ops.gemm_batched(q, self.qk_dim, self.w_uk_t, qa, self.row)
         ops.rope_heads(q, s.n_heads, self.qk_dim, s.head_dim, s.rot_dim, dims, cos, sin, qa, self.row, s.kv_rank)
         ol = ws.get("latent.ol", (n, s.n_heads * s.kv_rank), self.dtype)
@@ -147,6 +183,47 @@ class LatentAttention(Mixer):
             ops.gemm_batched(ol, s.kv_rank, self.w_uv, o, s.v_head_dim)
             if gate is not None:
                 ops.sigmoid_gate(o, gate)
+        stream(step).add_product(o, self.w_o, x_accum)
+
+
+    def _expanded_prompt(self, step, q, first, cos, sin, dims, cache, x_accum) -> None:
+        """A prompt step in the expanded form.  The cache rows the step's queries see (its own tokens, which
+        ``latent_prepare`` has appended, and up to window - 1 before them per sequence) are gathered into a
+        dense matrix in scratch-page order, one product turns them into every head's key and value, the
+        append kernel lays those out as pages of keys and transposed values, and the attention kernel for
+        separate heads runs over them with a block table of scratch pages.  Nothing of it is kept."""
+        s = self.spec
+        n, H, D = step.n_tokens, s.n_heads, self.qk_dim
+        ws = step.workspace
+        page = cache.k.shape[1]
+        span = s.window if s.window is not None else step.max_len
+        pages = sum(min((c + span) // page + 2, step.max_len // page + 1) for c in step.new_counts)
+        width = cache.block_table.shape[1]
+        table = ws.get("latent.x.table", (len(step.new_counts), width), torch.int32)
+        plan = ws.get("latent.x.plan", (4, pages), torch.int32)
+        ops.latent_window_plan(step.cu_seqlens, step.token_pos, cache.block_table, s.window, page, table, plan)
+        rows = ws.get("latent.x.rows", (pages * page, self.row), self.dtype)
+        ops.latent_window_gather(cache.k, plan, rows)
+        kv = ws.get("latent.x.kv", (pages * page, 2 * H * D), self.dtype)
+        ops.gemm(rows, self.w_expand, kv, workspace=ws.scratch())
+        ks = ws.get("latent.x.k", (pages, H, page, D), self.dtype)
+        vs = ws.get("latent.x.v", (pages, H, D, page), self.dtype)
+        if self._ident is None or self._ident[0].numel() < pages * page:
+            dev = kv.device
+            self._ident = (torch.arange(pages * page, dtype=torch.int32, device=dev),
+                           torch.zeros(pages * page, dtype=torch.int32, device=dev),
+                           torch.arange(pages, dtype=torch.int32, device=dev).view(1, pages))
+        pos_id, seq_id, table_id = self._ident
+        ops.qk_norm_rope_append(kv, 0, H, D, None, None, 1.0, None, None, 0, None, ks, vs, table_id[:, :pages].contiguous(),
+                                seq_id[:pages * page], pos_id[:pages * page], write_kv=True)
+        qf = ws.get("latent.x.q", (n, H * D), self.dtype)
+        ops.rope_heads(q, H, D, s.head_dim, s.rot_dim, dims, cos, sin, qf, D, 0, lead=s.head_dim)
+        of = ws.get("latent.x.o", (n, H * D), self.dtype)
+        ops.attention(qf, of, ks, vs, table, step.token_seq, step.token_pos, H, H, D, s.scale, s.window,
+                      workspace=ws.scratch(), cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
+                      max_len=step.max_len)
+        o = ws.get("latent.o", (n, self.o_dim), self.dtype)
+        ops.gate_heads(of, D, first[:, s.q_rank + self.row:] if s.gate else None, o, H, s.v_head_dim)
         stream(step).add_product(o, self.w_o, x_accum)
 
 

@@ -119,6 +119,9 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
         proj.shape[0] * sum(a[:3]) * 6, proj.shape[0] * sum(a[:3]) * 4)),
     "rope_heads": ("rotation of the queries' part", lambda q, n_heads, head_stride, offset, rot_part, *a, **kw: (
         q.shape[0] * n_heads * rot_part * 6, q.shape[0] * n_heads * rot_part * 3)),
+    "latent_window_plan": ("expanded prompt: plan of the visible rows", _tensor_args_cost(skip=(2,))),
+    "latent_window_gather": ("expanded prompt: gather of the visible rows", lambda cache, plan, out: (2 * _nbytes(out), 0)),
+    "gate_heads": ("output gate", lambda x, x_stride, gate, out, n_heads, n: (2 * _nbytes(out) + out.numel() * 4, 4 * out.numel())),
     "sigmoid_gate": ("output gate", lambda y, gate: (2 * _nbytes(y) + y.numel() * 4, 4 * y.numel())),
     "splitk_reduce": ("sum of K pieces", _tensor_args_cost()),
     "argmax": ("argmax", _tensor_args_cost()),

@@ -118,6 +118,29 @@ def test_portions_given_by_the_caller(models, name):
     assert helpers.per_position(torch.cat(out), ref) < 1e-4
 
 
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-4), ("bfloat16", 6e-2)])
+def test_long_portions_on_top_of_a_cache_with_unequal_starts(models, dtype, tol):
+    """Prompt steps of several hundred tokens (in bfloat16 the latent layers then expand keys and values per
+    head for what the step sees): on top of cached positions that the windows reach back into, and two
+    sequences with different first positions in one step."""
+    from rocml_amd.engine import StepEntry
+    path, cfg, tensors = models["Q"]
+    engine = _engine(path, dtype)
+    a, b = helpers.random_tokens(760, cfg["vocab"], 61), helpers.random_tokens(300, cfg["vocab"], 62)
+    ref_a, ref_b = plain.forward(cfg, tensors, a), plain.forward(cfg, tensors, b)
+    sa, sb = engine.new_sequence(), engine.new_sequence()
+    out_a = [engine.step([StepEntry(sa, a[:90], list(range(90)))]).cpu()]              # a short first portion
+    out_a.append(engine.step([StepEntry(sa, a[90:390], list(range(300)))]).cpu())      # 300 tokens on top of 90
+    both = engine.step([StepEntry(sa, a[390:], list(range(370))), StepEntry(sb, b[:280], list(range(280)))]).cpu()
+    out_a.append(both[:370])
+    out_b = [both[370:], engine.step([StepEntry(sb, b[280:], list(range(20)))]).cpu()]
+    engine.release(sa)
+    engine.release(sb)
+    assert helpers.per_position(torch.cat(out_a), ref_a) < tol
+    assert helpers.per_position(torch.cat(out_b), ref_b) < tol
+    engine.cache.check()
+
+
 def test_pages_are_given_back_and_used_again(models):
     """A cache far smaller than the tokens that pass through it: windows and blocks give their pages
     back while a request runs, and ended requests give back the rest."""
