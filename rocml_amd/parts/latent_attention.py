@@ -12,7 +12,10 @@ and nothing per head.  The attention never expands the keys: since
 every head asks one shared key/value "head" whose keys are the cache rows ``[c_j, k_r(j)]`` and
 whose values are the first ``kv_rank`` numbers of the same rows, with the query
 ``[W_uk,a^T q_a^n, q_a^r]``; the head's output is ``W_uv,a`` times what the attention returns.
-Both small products run once per token and head, whatever the number of keys.
+Both small products run once per token and head, whatever the number of keys.  Long prompt steps in
+bfloat16 take the other road (``_expanded_prompt``): keys and values per head, expanded for the
+positions the step sees, which costs a third of the operations per (query, key) pair at the usual
+sizes; the cache is the same rows either way.
 
 Launches of a step: one product for the three projections of ``h`` (query latent, key/value
 latent with its rotated part, output gate), one kernel that norms both latents, rotates and
