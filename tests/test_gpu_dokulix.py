@@ -237,3 +237,19 @@ def test_command_line_runs_the_design(models, capsys):
     assert main(["generate", "--model", "dokulix-tiny", "--prompt-ids", "1 2 3", "-n", "4", "--ctx", "64", "--batch", "1"]) == 0
     assert len(capsys.readouterr().out.strip().splitlines()[-1].split()) == 4
     assert main(["models"]) == 0 and "dokulix-2b" in capsys.readouterr().out
+
+
+@pytest.mark.parametrize("name,length", [("Q", 300), ("P", 150)])
+def test_prompt_steps_of_one_shape_are_replayed(models, name, length):
+    """The second prompt step of a shape is recorded as a graph and later ones replayed: four different
+    prompts of one length (for Q long enough for the expanded form), each against the plain implementation,
+    with decode steps between them."""
+    path, cfg, tensors = models[name]
+    engine = _engine(path, "bfloat16")
+    assert engine.model.prompt_graph_safe and engine.use_graphs
+    for k in range(4):
+        p = helpers.random_tokens(length + 3, cfg["vocab"], 1000 + k)
+        ref = plain.forward(cfg, tensors, p)
+        got = helpers.run_tail_by_one(engine, p, 3)
+        assert helpers.per_position(got, ref) < TOL["bfloat16"], f"prompt {k}"
+    assert any(key[0] == "prompt" and entry[1] is not None for key, entry in engine._graphs.items()), "a prompt shape was recorded"
