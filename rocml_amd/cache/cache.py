@@ -30,7 +30,7 @@ import numpy as np
 import torch
 
 from ..errors import CacheFullError, MemoryBudgetError, RocmlError
-from ..parts.base import KVCacheRequest, LatentCacheRequest, StateRequest
+from ..parts.base import CompositeRequest, KVCacheRequest, LatentCacheRequest, StateRequest
 
 PAGE_SIZE = 64
 
@@ -341,6 +341,7 @@ class CacheLineView:
     block_table: Optional[torch.Tensor] = None  # [B, width] int32 on the device, per step
     state: Optional[torch.Tensor] = None        # [slots, *shape]
     slots: Optional[torch.Tensor] = None        # [B] int32 on the device, per step
+    parts: Optional[tuple] = None               # a composite request's views, in the request's order (None where a part asked for nothing)
 
 
 # Memory left free beside the cache for activations and the runtime: the reference keeps
@@ -356,11 +357,22 @@ def _geometry(max_tokens: int, dtype, device, max_seqs: Optional[int], page_size
                     max_seqs=max_seqs, step_tokens=step_tokens, dtype=dtype, device=device)
 
 
-def _by_request(requests: Sequence[Optional[object]]) -> Dict[object, List[int]]:
-    by_request: Dict[object, List[int]] = {}
+def _leaves(key: tuple, req):
+    """The plain requests inside ``req`` with their place: ``(entry, part, part of part, ...)``."""
+    if isinstance(req, CompositeRequest):
+        for j, part in enumerate(req.parts):
+            yield from _leaves(key + (j,), part)
+    elif req is not None:
+        yield key, req
+
+
+def _by_request(requests: Sequence[Optional[object]]) -> Dict[object, List[tuple]]:
+    """Cache lines with one request, each named by its schedule entry and, inside a composite
+    request, the part's place."""
+    by_request: Dict[object, List[tuple]] = {}
     for entry, req in enumerate(requests):
-        if req is not None:
-            by_request.setdefault(req, []).append(entry)
+        for key, leaf in _leaves((entry,), req):
+            by_request.setdefault(leaf, []).append(key)
     return by_request
 
 
@@ -412,7 +424,8 @@ class Cache:
         self.slots = SlotAllocator(self.max_seqs)
         self.lengths: Dict[int, int] = {}
         self.groups: List[CacheGroup] = []
-        self._line_of: Dict[int, Tuple[CacheGroup, int]] = {}
+        self._line_of: Dict[tuple, Tuple[CacheGroup, int]] = {}
+        self._requests = list(requests)
         for req, entries in _by_request(requests).items():
             kind = _group_type(req)
             tag = kind.__name__.replace("Group", "").lower()
@@ -527,11 +540,25 @@ class Cache:
     def table_width(self, slots: Sequence[int]) -> int:
         return max([1] + [len(g.page_table(s)) for g in self.kv_groups for s in slots])
 
-    def line(self, entry: int) -> Tuple[object, int]:
-        return self._line_of[entry]
+    def line(self, entry: int, *part: int) -> Tuple[object, int]:
+        """Group and line of a schedule entry's storage (of part ``part`` of a composite request)."""
+        return self._line_of[(entry,) + tuple(part)]
 
     def has_line(self, entry: int) -> bool:
-        return entry in self._line_of
+        return any(True for _ in _leaves((entry,), self._requests[entry]))
+
+    def view(self, entry: int, step) -> Optional["CacheLineView"]:
+        """What the mixer of schedule entry ``entry`` sees in this step: its line's view, or for a
+        composite request a view whose ``parts`` are the parts' views."""
+        def build(key: tuple, req):
+            if req is None:
+                return None
+            if isinstance(req, CompositeRequest):
+                return CacheLineView(group=None, line=-1,
+                                     parts=tuple(build(key + (j,), part) for j, part in enumerate(req.parts)))
+            group, line = self._line_of[key]
+            return group.view(line, step)
+        return build((entry,), self._requests[entry])
 
     def check(self) -> None:
         for g in self.groups:

@@ -111,6 +111,13 @@ def _register_builtin() -> None:
         to_spec=lambda cfg: cfg.to_model_spec(),
         checkpoint_names=dokulix.checkpoint_names,
         unused_tensors=dokulix.unused_tensors))
+    from . import felovik
+    register_architecture(Architecture(
+        name=felovik.ARCHITECTURE,
+        read_config=felovik.FelovikConfig.from_dict,
+        to_spec=lambda cfg: cfg.to_model_spec(),
+        checkpoint_names=felovik.checkpoint_names,
+        unused_tensors=felovik.unused_tensors))
 
 
 _register_builtin()

@@ -21,11 +21,13 @@ from typing import Any, Optional, Tuple
 @dataclass(frozen=True)
 class NormSpec:
     """Root-mean-square norm over the last ``size`` values with a gain vector.  ``unit_offset``:
-    the stored weight lies around zero and the gain is one plus it."""
+    the stored weight lies around zero and the gain is one plus it.  ``learned`` false: the norm
+    has no weight, the values are only divided by their root mean square."""
     size: int
     eps: float
     kind: str = "rmsnorm"
     unit_offset: bool = False
+    learned: bool = True
 
 
 @dataclass(frozen=True)
@@ -51,7 +53,9 @@ class AttentionSpec:
     of so many, counted from position 0, and a query sees the keys of its own block up to itself.
     ``distance_slopes``: one number per query head; ``slope * (i - j)`` is taken off the score of
     query ``i`` and key ``j``.  ``sink``: the softmax's denominator has one more term, ``exp(0)``,
-    which has no value."""
+    which has no value.  ``q_temp``: ``(coef, every)``; the query at position ``p`` is multiplied by
+    ``1 + coef * ln(floor((p + 1) / every) + 1)`` after its norm.  ``gate``: the concatenated heads
+    are multiplied by ``sigmoid(W_g h)`` of the mixer's input before the output projection."""
     hidden: int
     n_heads: int
     n_kv_heads: int
@@ -66,6 +70,8 @@ class AttentionSpec:
     chunk: Optional[int] = None
     distance_slopes: Optional[Tuple[float, ...]] = None
     sink: bool = False
+    q_temp: Optional[Tuple[float, int]] = None
+    gate: bool = False
 
 
 @dataclass(frozen=True)
@@ -97,11 +103,67 @@ class LatentAttentionSpec:
 
 @dataclass(frozen=True)
 class GatedMlpSpec:
-    """Dense gated feed-forward: ``down(act(gate(x)) * up(x))``."""
+    """Dense gated feed-forward: ``down(act(g) * (u + up_offset))`` with ``g = gate(x)``,
+    ``u = up(x)``.  ``limit``: ``g`` is cut off above at ``limit`` and ``u`` is held inside
+    ``[-limit, limit]`` before anything else."""
     hidden: int
     intermediate: int
     activation: str = "silu"
     kind: str = "gated_mlp"
+    limit: Optional[float] = None
+    up_offset: float = 0.0
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """A feed-forward of ``n_experts`` small gated feed-forwards (``down(act(gate x) * up x)``,
+    no biases) of which each token uses ``top``.  The router's logits ``W_router h`` and their
+    softmax over all experts are 32-bit.  ``groups``: ``(count, keep)``; the experts form ``count``
+    equal groups of neighbours, a group's score is its largest expert score, and only experts of
+    the ``keep`` best groups can be chosen.  The chosen experts' scores, divided by their sum plus
+    ``sum_eps``, weight their outputs."""
+    hidden: int
+    n_experts: int
+    top: int
+    intermediate: int
+    activation: str = "silu"
+    groups: Optional[Tuple[int, int]] = None
+    sum_eps: float = 1e-20
+    kind: str = "routed_experts"
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    """A recurrence with one scalar decay per head (state-space duality): the input projection gives
+    ``[z: inner | x: inner | B: groups * state | C: groups * state | dt: n_heads]`` with
+    ``inner = n_heads * head_dim``; x, B and C pass a causal convolution of ``conv`` taps per channel
+    (with bias) and silu; ``dt <- softplus(dt + dt_bias)``; per head (head ``a`` uses group
+    ``a // (n_heads / groups)``) ``S <- exp(-exp(A_log) dt) S + dt B x^T``, ``y = S^T C + D x``;
+    ``y * silu(z)`` is normed in ``norm_groups`` equal parts and projected back.  The state
+    (``state x head_dim`` per head) and the convolution's last ``conv - 1`` inputs are 32-bit and
+    live per sequence."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int
+    eps: float
+    kind: str = "state_space"
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """A set of mixers that all run on one input.  The result is
+    ``weight * sum_b norm_b(out_b)``: each branch's output is normed over the model width with a
+    gain of its own.  ``branches`` are ``(name, mixer spec)`` pairs; a branch's parameters and
+    its output norm carry its name."""
+    hidden: int
+    branches: Tuple[Tuple[str, Any], ...]
+    weight: float
+    eps: float
+    kind: str = "parallel"
 
 
 @dataclass(frozen=True)
@@ -111,6 +173,17 @@ class TokenTableSpec:
     hidden: int
     scale: float = 1.0
     kind: str = "token_table"
+
+
+@dataclass(frozen=True)
+class TokenPositionTableSpec:
+    """The model's input: a token's row of a ``[vocab, hidden]`` table times ``scale`` plus the
+    row of its position in a learned ``[max_positions, hidden]`` table (not scaled)."""
+    vocab: int
+    hidden: int
+    max_positions: int
+    scale: float = 1.0
+    kind: str = "token_position_table"
 
 
 @dataclass(frozen=True)
@@ -130,12 +203,15 @@ class BlockSpec:
 
     ``arrangement`` names how they are wired; ``pre_norm`` is
     ``x += mixer(norm(x)); x += ffn(norm(x))``.  ``ffn`` (and then ``ffn_norm``) may be None:
-    the layer is its mixer alone."""
+    the layer is its mixer alone.  ``post_norm`` is
+    ``x <- norm(residual_scale * x + mixer(x)); x <- norm(residual_scale * x + ffn(x))``: the
+    sublayers read the stream itself and the norms come after the sums."""
     mixer: Any
     ffn: Any
     mixer_norm: NormSpec
     ffn_norm: Optional[NormSpec]
     arrangement: str = "pre_norm"
+    residual_scale: float = 1.0
 
 
 @dataclass(frozen=True)

@@ -3,7 +3,7 @@
 The reference compiles every kernel source at build time with ``hipcc --genco
 --offload-arch=... -O3`` and fails with the compiler's output
 (rocml-kernels/build.rs:10-59).  Here each family (``elementwise``, ``gemm``,
-``attention``, ``sampling``) becomes ``_build/lib<family>.so`` next to the sources;
+``attention``, ``sampling``, ``recurrent``, ``moe``) becomes ``_build/lib<family>.so`` next to the sources;
 a family is compiled when it is first needed and no library built from the present
 sources is there (a hash of the sources and flags is kept beside each library), so a
 fresh checkout works without a build step and an edited kernel is never run from an
@@ -25,7 +25,7 @@ from typing import Dict, Iterable, List
 from ..errors import ExtensionMissingError
 
 SRC_DIR = os.path.dirname(os.path.abspath(__file__))
-FAMILIES = ("elementwise", "gemm", "attention", "sampling")
+FAMILIES = ("elementwise", "gemm", "attention", "sampling", "recurrent", "moe")
 ARCH = "gfx950"
 # Packed 32-bit float instructions are switched off for all device code.
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",

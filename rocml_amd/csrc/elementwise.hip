@@ -11,29 +11,41 @@ constexpr int EW_BLOCK = 256;
 // ---- embedding -------------------------------------------------------------------
 // out[t, :] = float(table[ids[t], :]) * scale  (rocml-kernels/kernels/embedding.hip:6-18;
 // the reference has no scale, callers pass 1).
+// With a table of positions ([max_pos, hidden], same type): the row of the token's position is
+// added, not scaled.
 template <typename T>
 __global__ void embed_gather_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ out, int hidden, int vocab, float scale) {
+                                    float* __restrict__ out, int hidden, int vocab, float scale,
+                                    const T* __restrict__ pos_table, const int* __restrict__ positions, int max_pos) {
     int t = blockIdx.x;
     int id = ids[t];
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
     const T* row = table + (size_t)id * hidden;
     float* o = out + (size_t)t * hidden;
+    if (pos_table) {
+        int p = positions[t];
+        p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);
+        const T* prow = pos_table + (size_t)p * hidden;
+        for (int i = threadIdx.x; i < hidden; i += EW_BLOCK) o[i] = fmaf(Elem<T>::load(row + i), scale, Elem<T>::load(prow + i));
+        return;
+    }
     for (int i = threadIdx.x; i < hidden; i += EW_BLOCK) o[i] = Elem<T>::load(row + i) * scale;
 }
 
 ROCML_EXPORT int rocml_embed_gather(const void* table, int table_dtype, const int* ids, float* out,
                                     int n_tokens, int hidden, int vocab, float scale,
+                                    const void* pos_table, const int* positions, int max_pos,
                                     hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes T=%d H=%d V=%d",
                   n_tokens, hidden, vocab);
+    ROCML_REQUIRE(!pos_table || (positions && max_pos > 0), "embed_gather: a table of positions needs the positions");
     if (n_tokens == 0) return 0;
     if (table_dtype == ROCML_F32)
         embed_gather_kernel<float><<<n_tokens, EW_BLOCK, 0, stream>>>((const float*)table, ids, out,
-                                                                      hidden, vocab, scale);
+                                                                      hidden, vocab, scale, (const float*)pos_table, positions, max_pos);
     else if (table_dtype == ROCML_BF16)
         embed_gather_kernel<bf16_t><<<n_tokens, EW_BLOCK, 0, stream>>>((const bf16_t*)table, ids, out,
-                                                                       hidden, vocab, scale);
+                                                                       hidden, vocab, scale, (const bf16_t*)pos_table, positions, max_pos);
     else
         return rocml_fail("embed_gather: unknown dtype code %d", table_dtype);
     ROCML_CHECK_LAUNCH("embed_gather");
@@ -205,16 +217,20 @@ ROCML_EXPORT int rocml_rmsnorm(float* x, const float* gain, void* out, int out_d
 // (rocml-kernels/kernels/silu_mul.hip:12-20).  Gate and up halves lie side by side in a row.
 // With `interleaved` a row holds (gate_0, up_0, gate_1, up_1, ...), the order the fused product
 // epilogue wants its weight rows in.
-// act: 0 silu, 1 relu (max(g, 0)), 2 gelu with the tanh form 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))).
+// act: 0 silu, 1 relu (max(g, 0)), 2 gelu with the tanh form 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))),
+// 3 g sigmoid(1.702 g).
 __device__ __forceinline__ float gate_activation(float g, int act) {
     if (act == 1) return fmaxf(g, 0.f);
+    if (act == 3) return g / (1.0f + expf(-1.702f * g));      // g sigmoid(1.702 g)
     if (act == 2) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
     return g / (1.0f + expf(-g));
 }
 
+// limit > 0: g is cut off above at limit and u is held inside [-limit, limit] first; up_offset is
+// added to u (after the limit).
 template <typename TI, typename TO>
 __global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter,
-                              long long total, int interleaved, int act) {
+                              long long total, int interleaved, int act, float limit, float up_offset) {
     long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
     if (idx >= total) return;
     long long t = idx / inter;
@@ -222,22 +238,27 @@ __global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, i
     const TI* row = gu + (size_t)t * 2 * inter;
     float g = Elem<TI>::load(row + (interleaved ? 2 * i : i));
     float u = Elem<TI>::load(row + (interleaved ? 2 * i + 1 : inter + i));
-    Elem<TO>::store(out + idx, gate_activation(g, act) * u);
+    if (limit > 0.f) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+    }
+    Elem<TO>::store(out + idx, gate_activation(g, act) * (u + up_offset));
 }
 
 ROCML_EXPORT int rocml_swiglu(const void* gu, int in_dtype, void* out, int out_dtype, int n_tokens,
-                              int inter, int interleaved, int act, hipStream_t stream) {
+                              int inter, int interleaved, int act, float limit, float up_offset, hipStream_t stream) {
     ROCML_REQUIRE(n_tokens >= 0 && inter > 0, "swiglu: bad sizes T=%d I=%d", n_tokens, inter);
-    ROCML_REQUIRE(act >= 0 && act <= 2, "swiglu: unknown activation %d (0 silu, 1 relu, 2 gelu_tanh)", act);
+    ROCML_REQUIRE(act >= 0 && act <= 3, "swiglu: unknown activation %d (0 silu, 1 relu, 2 gelu_tanh, 3 sigmoid_1702)", act);
+    ROCML_REQUIRE(limit >= 0.f, "swiglu: the limit must not be negative (0: none)");
     long long total = (long long)n_tokens * inter;
     if (total == 0) return 0;
     int grid = ceil_div(total, EW_BLOCK);
     if (in_dtype == ROCML_F32 && out_dtype == ROCML_F32)
-        swiglu_kernel<float, float><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (float*)out, inter, total, interleaved, act);
+        swiglu_kernel<float, float><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (float*)out, inter, total, interleaved, act, limit, up_offset);
     else if (in_dtype == ROCML_F32 && out_dtype == ROCML_BF16)
-        swiglu_kernel<float, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (bf16_t*)out, inter, total, interleaved, act);
+        swiglu_kernel<float, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const float*)gu, (bf16_t*)out, inter, total, interleaved, act, limit, up_offset);
     else if (in_dtype == ROCML_BF16 && out_dtype == ROCML_BF16)
-        swiglu_kernel<bf16_t, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, interleaved, act);
+        swiglu_kernel<bf16_t, bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, total, interleaved, act, limit, up_offset);
     else
         return rocml_fail("swiglu: unsupported dtype pair in=%d out=%d", in_dtype, out_dtype);
     ROCML_CHECK_LAUNCH("swiglu");
@@ -281,6 +302,11 @@ ROCML_EXPORT int rocml_rope_table(const int* pos, const double* inv_freq, float*
 // reference's separate scatter).  Cache layout: keys [page, Hkv, page_size, D], values
 // transposed inside a page [page, Hkv, D, page_size] (what the MFMA attention kernels read).
 constexpr int QK_MAX_PER_LANE = 8;   // D <= 512
+
+// A query's stretch with its position: 1 + coef * ln(floor((p + 1) / every) + 1); every = 0: none.
+__device__ __forceinline__ float query_temperature(int pos, float coef, int every) {
+    return every > 0 ? 1.0f + coef * logf((float)((pos + 1) / every + 1)) : 1.0f;
+}
 constexpr int QK_WAVES = EW_BLOCK / WAVE;
 
 // LOCAL_PAIR: the whole head is rotated and a lane holds at least two values, so both values of a
@@ -293,7 +319,9 @@ __global__ void qk_norm_rope_append_kernel(
     TO* __restrict__ q_out, TO* __restrict__ kcache, TO* __restrict__ vcache,
     const int* __restrict__ block_table, int bt_width, const int* __restrict__ token_seq,
     const int* __restrict__ token_pos, int page_size, int write_kv, int n_splits, long long split_stride,
-    int rows_per_token, int pairing, int first_row, const float* __restrict__ bias, int dv) {
+    int rows_per_token, int pairing, int first_row, const float* __restrict__ bias, int dv,
+    float qt_coef, int qt_every) {
+    // qt_coef, qt_every: the queries' stretch with their position (after the norm); every = 0: none.
     // bias (may be null): one number per column of the packed row, added to the projection's sums.
     // dv: the size of a value head; the value rows start behind the Hq + Hkv rows of d numbers.
     extern __shared__ float stage[];   // [QK_WAVES][d]
@@ -340,6 +368,11 @@ __global__ void qk_norm_rope_append_kernel(
             int e = lane + j * WAVE;
             if (e < d) v[j] = v[j] * inv * gain[e];
         }
+    }
+    if (qt_every > 0 && kind == 0) {
+        float temp = query_temperature(token_pos[t], qt_coef, qt_every);
+#pragma unroll
+        for (int j = 0; j < QK_PER_LANE; ++j) v[j] *= temp;
     }
     bool rotate = cos_t != nullptr && kind != 2;
     if (LOCAL_PAIR) {
@@ -426,7 +459,7 @@ qk_norm_rope_rows_kernel(
     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     TO* __restrict__ q_out, TO* __restrict__ kcache, const int* __restrict__ block_table, int bt_width,
     const int* __restrict__ token_seq, const int* __restrict__ token_pos, int page_size, int rows_per_token,
-    int first_row, const float* __restrict__ bias) {
+    int first_row, const float* __restrict__ bias, float qt_coef, int qt_every) {
     constexpr int HJ = QK_PER_LANE / 2;
     int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
     long long total = (long long)n_tokens * rows_per_token;
@@ -464,6 +497,11 @@ qk_norm_rope_rows_kernel(
             float inv = 1.0f / sqrtf(wave_sum(ss) / (float)d + eps);
 #pragma unroll
             for (int j = 0; j < QK_PER_LANE; ++j) v[i][j] = v[i][j] * inv * gain[lane + j * WAVE];
+        }
+        if (qt_every > 0 && is_q) {
+            float temp = query_temperature(token_pos[tok[i]], qt_coef, qt_every);
+#pragma unroll
+            for (int j = 0; j < QK_PER_LANE; ++j) v[i][j] *= temp;
         }
         if (cos_t) {
 #pragma unroll
@@ -534,9 +572,12 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     const float* k_gain, float eps, const float* cos_t, const float* sin_t, int rot, int pairing, void* q_out,
     void* kcache, void* vcache, int out_dtype, const int* block_table, int bt_width,
     const int* token_seq, const int* token_pos, int page_size, int write_kv, int n_splits,
-    long long split_stride, const float* bias, int dv, hipStream_t stream) {
+    long long split_stride, const float* bias, int dv, float qt_coef, int qt_every, hipStream_t stream) {
     // bias (may be null): [ld] numbers added to the projection's sums; dv (0: d): value head size.
+    // qt_coef, qt_every: a query at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1)
+    // after its norm (every = 0: not).
     if (dv <= 0) dv = d;
+    ROCML_REQUIRE(qt_every >= 0, "qk_norm_rope_append: the query stretch's period must not be negative");
     ROCML_REQUIRE(n_tokens >= 0 && (hq > 0 || (hq == 0 && !q_out)) && hkv > 0 && d > 0, "qk_norm_rope_append: bad sizes");
     ROCML_REQUIRE(dv <= QK_MAX_PER_LANE * WAVE, "qk_norm_rope_append: value head size %d exceeds %d", dv,
                   QK_MAX_PER_LANE * WAVE);
@@ -573,12 +614,12 @@ ROCML_EXPORT int rocml_qk_norm_rope_append(
     qk_norm_rope_append_kernel<TI, TO, N, LP><<<grid, EW_BLOCK, lds, stream>>>(                 \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, cos_t, sin_t, rot,       \
         (TO*)q_out, (TO*)kcache, (TO*)vcache, block_table, bt_width, token_seq, token_pos,      \
-        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row, bias, dv)
+        page_size, write_kv, n_splits, split_stride, rows_per_token, pairing, first_row, bias, dv, qt_coef, qt_every)
 #define LAUNCH_ROWS(TI, TO, N)                                                                  \
     qk_norm_rope_rows_kernel<TI, TO, N, MANY><<<grid, EW_BLOCK, 0, stream>>>(                   \
         (const TI*)qkv, ld, n_tokens, hq, hkv, d, q_gain, k_gain, eps, rot ? cos_t : nullptr,   \
         rot ? sin_t : nullptr, (TO*)q_out, (TO*)kcache, block_table, bt_width, token_seq,       \
-        token_pos, page_size, rows_per_token, first_row, bias)
+        token_pos, page_size, rows_per_token, first_row, bias, qt_coef, qt_every)
 #define LAUNCH(TI, TO)                                                                          \
     {                                                                                           \
         if (many_rows) { if (per_lane == 2) LAUNCH_ROWS(TI, TO, 2); else LAUNCH_ROWS(TI, TO, 4); } \
@@ -928,5 +969,102 @@ ROCML_EXPORT int rocml_gate_heads(const void* x, int dtype, int ldx, int x_strid
     else if (dtype == ROCML_BF16) gate_heads_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>((const bf16_t*)x, ldx, x_stride, g, ldg, (bf16_t*)out, n_heads, n, total);
     else return rocml_fail("gate_heads: unknown dtype code %d", dtype);
     ROCML_CHECK_LAUNCH("gate_heads");
+    return 0;
+}
+
+// ---- norm after the sum ----------------------------------------------------------
+// x[t, :] <- rms(alpha * x[t, :] + c * sum_b f_b(y_b[t, :])) * gain (without a gain: the sum
+// itself, not normed), all in 32-bit, with
+// f_b(y) = y / sqrt(mean(y^2) + eps) * gain_b for a branch with a gain and f_b(y) = y without.
+// It is the layer wiring "the sublayer reads the stream, the norm comes after the sum", and with two
+// or more branches also the sum of sublayers that ran side by side on the same input, each normed
+// over the width first.  x is rewritten in place; `copy` (may be null) gets the new x in another
+// type, for the products that read it next.  One block per row.
+constexpr int SN_MAX_BRANCHES = 4;
+struct SumNormBranches {
+    const float* y[SN_MAX_BRANCHES];
+    const float* gain[SN_MAX_BRANCHES];
+    int n;
+};
+
+template <typename TC>
+__global__ void __launch_bounds__(EW_BLOCK)
+sum_norm_kernel(float* __restrict__ x, SumNormBranches br, float alpha, float c, const float* __restrict__ gain,
+                float eps, int n, TC* __restrict__ copy) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    size_t row = (size_t)blockIdx.x * n;
+    float inv[SN_MAX_BRANCHES];
+#pragma unroll
+    for (int b = 0; b < SN_MAX_BRANCHES; ++b) {
+        inv[b] = 1.f;
+        if (b < br.n && br.gain[b]) {
+            float ss = 0.f;
+            for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
+                float v = br.y[b][row + i];
+                ss = fmaf(v, v, ss);
+            }
+            inv[b] = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+        }
+    }
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) {
+        float sum = 0.f;
+#pragma unroll
+        for (int b = 0; b < SN_MAX_BRANCHES; ++b)
+            if (b < br.n) {
+                float v = br.y[b][row + i];
+                sum += br.gain[b] ? v * inv[b] * br.gain[b][i] : v;
+            }
+        float s = alpha != 0.f ? fmaf(alpha, x[row + i], c * sum) : c * sum;      // alpha = 0: x is not read
+        x[row + i] = s;
+        ss = fmaf(s, s, ss);
+    }
+    if (!gain && !copy) return;
+    float r = gain ? 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps) : 1.f;
+    for (int i = threadIdx.x; i < n; i += EW_BLOCK) {       // a thread reads back what it wrote itself
+        float v = gain ? x[row + i] * r * gain[i] : x[row + i];
+        x[row + i] = v;
+        if (copy) Elem<TC>::store(copy + row + i, v);
+    }
+}
+
+ROCML_EXPORT int rocml_sum_norm(float* x, int n_rows, int n, float alpha, float c, int n_branches,
+                                const float* const* ys, const float* const* gains, const float* gain, float eps,
+                                void* copy, int copy_dtype, hipStream_t stream) {
+    ROCML_REQUIRE(n_rows >= 0 && n > 0, "sum_norm: bad sizes rows=%d n=%d", n_rows, n);
+    ROCML_REQUIRE(n_branches >= 1 && n_branches <= SN_MAX_BRANCHES, "sum_norm: %d branches (1 to %d)", n_branches, SN_MAX_BRANCHES);
+    ROCML_REQUIRE(x && ys && gains, "sum_norm: missing arguments");
+    if (n_rows == 0) return 0;
+    SumNormBranches br{};
+    br.n = n_branches;
+    for (int b = 0; b < n_branches; ++b) {
+        ROCML_REQUIRE(ys[b], "sum_norm: branch %d has no values", b);
+        br.y[b] = ys[b];
+        br.gain[b] = gains[b];
+    }
+    if (!copy || copy_dtype == ROCML_F32)
+        sum_norm_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, br, alpha, c, gain, eps, n, (float*)copy);
+    else if (copy_dtype == ROCML_BF16)
+        sum_norm_kernel<bf16_t><<<n_rows, EW_BLOCK, 0, stream>>>(x, br, alpha, c, gain, eps, n, (bf16_t*)copy);
+    else return rocml_fail("sum_norm: unknown dtype code %d", copy_dtype);
+    ROCML_CHECK_LAUNCH("sum_norm");
+    return 0;
+}
+
+// ---- a copy of 32-bit values in another type -----------------------------------------
+template <typename TO>
+__global__ void convert_kernel(const float* __restrict__ x, TO* __restrict__ out, long long total) {
+    long long idx = (long long)blockIdx.x * EW_BLOCK + threadIdx.x;
+    if (idx < total) Elem<TO>::store(out + idx, x[idx]);
+}
+
+ROCML_EXPORT int rocml_convert(const float* x, void* out, int out_dtype, long long total, hipStream_t stream) {
+    ROCML_REQUIRE(total >= 0, "convert: negative size");
+    if (total == 0) return 0;
+    int grid = ceil_div(total, EW_BLOCK);
+    if (out_dtype == ROCML_F32) convert_kernel<float><<<grid, EW_BLOCK, 0, stream>>>(x, (float*)out, total);
+    else if (out_dtype == ROCML_BF16) convert_kernel<bf16_t><<<grid, EW_BLOCK, 0, stream>>>(x, (bf16_t*)out, total);
+    else return rocml_fail("convert: unknown dtype code %d", out_dtype);
+    ROCML_CHECK_LAUNCH("convert");
     return 0;
 }

@@ -50,6 +50,16 @@ class DecoderModel:
         self.prompt_graph_safe = self.graph_safe and all(getattr(part, "prompt_graph_safe", False)
                                                          for part in [self.embedding, self.head] + self.blocks)
 
+    def kernel_families(self):
+        """The kernel libraries this model's steps launch from: the ones every model needs and those
+        its parts name (``kernel_families``), so that a fresh checkout compiles what the model uses."""
+        families = list(ops.MODEL_FAMILIES)
+        for part in [self.embedding, self.head] + self.blocks:
+            for f in getattr(part, "kernel_families", ()):
+                if f not in families:
+                    families.append(f)
+        return tuple(families)
+
     @property
     def embed(self) -> Optional[torch.Tensor]:
         """The embedding's table (None before weights are bound or if it has none)."""
@@ -168,10 +178,7 @@ class DecoderModel:
         self.embedding.forward(step, x)
         for i, entry in enumerate(s.schedule):
             owner = i if entry.reads_cache_of is None else entry.reads_cache_of
-            view = None
-            if cache.has_line(owner):
-                group, line = cache.line(owner)
-                view = group.view(line, step)
+            view = cache.view(owner, step) if cache.has_line(owner) else None
             block = self.blocks[entry.layer]
             if entry.offset_row is not None:
                 # (sums that a product left for the next norm may still be missing from x: additions commute)

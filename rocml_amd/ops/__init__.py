@@ -27,12 +27,12 @@ _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
 _SIGNATURES = {
     "elementwise": {
-        "rocml_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _F, _P],
+        "rocml_embed_gather": [_P, _I, _P, _P, _I, _I, _I, _F, _P, _P, _I, _P],
         "rocml_rmsnorm": [_P, _P, _P, _I, _P, _I, _I, _F, _P, _I, _LL, _P],
-        "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _I, _I, _P],
+        "rocml_swiglu": [_P, _I, _P, _I, _I, _I, _I, _I, _F, _F, _P],
         "rocml_rope_table": [_P, _P, _P, _P, _I, _I, _P],
         "rocml_qk_norm_rope_append": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _I, _I, _P, _P, _P,
-                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _P],
+                                      _I, _P, _I, _P, _P, _I, _I, _I, _LL, _P, _I, _F, _I, _P],
         "rocml_add_into": [_P, _P, _I, _LL, _P],
         "rocml_add_row_vector": [_P, _P, _I, _I, _P],
         "rocml_latent_prepare": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _P],
@@ -41,6 +41,19 @@ _SIGNATURES = {
         "rocml_latent_window_gather": [_P, _I, _I, _I, _P, _I, _P, _P],
         "rocml_gate_heads": [_P, _I, _I, _I, _P, _I, _P, _I, _I, _I, _P],
         "rocml_sigmoid_gate": [_P, _I, _P, _I, _I, _I, _P],
+        "rocml_sum_norm": [_P, _I, _I, _F, _F, _I, _P, _P, _P, _F, _P, _I, _P],
+        "rocml_convert": [_P, _P, _I, _LL, _P],
+    },
+    "recurrent": {
+        "rocml_causal_conv": [_P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _P, _I, _P, _I, _P],
+        "rocml_ssd_scan": [_P, _I, _P, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P, _I, _I, _I, _I, _P],
+        "rocml_gated_part_norm": [_P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
+    },
+    "moe": {
+        "rocml_moe_route": [_P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+        "rocml_moe_plan": [_P, _I, _I, _P, _P, _P, _P, _P, _I, _P],
+        "rocml_moe_gemm": [_P, _I, _I, _I, _P, _I, _P, _P, _I, _LL, _I, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P],
+        "rocml_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
     },
     "gemm": {
         "rocml_gemm": [_P, _I, _I, _P, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _LL, _P, _I, _F, _I, _P],
@@ -82,7 +95,8 @@ def library(family: str) -> ctypes.CDLL:
     return lib
 
 
-MODEL_FAMILIES = ("elementwise", "gemm", "attention")   # what a model's step needs; sampling comes with generation
+MODEL_FAMILIES = ("elementwise", "gemm", "attention")   # what every model's step needs; sampling comes with generation,
+                                                        # and a part with kernels of another family names it (``kernel_families``)
 
 
 def prepare(families=tuple(_SIGNATURES)) -> None:
@@ -157,8 +171,18 @@ def _want(t: torch.Tensor, dtype: torch.dtype, what: str) -> None:
 
 
 # ---- elementwise ---------------------------------------------------------------------
-def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
-    _dev(table, ids, out)
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0,
+                 pos_table: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None) -> None:
+    """``out[t] = table[ids[t]] * scale`` and, with a table of positions ``[max_positions, hidden]``
+    of the same type, ``+ pos_table[positions[t]]`` (not scaled)."""
+    _dev(table, ids, out, pos_table, positions)
+    max_pos = 0
+    if pos_table is not None:
+        if positions is None or positions.numel() != ids.numel() or pos_table.dtype != table.dtype \
+                or pos_table.dim() != 2 or pos_table.shape[1] != table.shape[1]:
+            raise KernelError("a table of positions needs one position per token and the token table's type and width")
+        _want(positions, torch.int32, "positions")
+        max_pos = pos_table.shape[0]
     _want(ids, torch.int32, "token ids")
     _want(out, torch.float32, "embedding output")
     vocab, hidden = table.shape
@@ -166,7 +190,8 @@ def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scal
     if out.shape != (n, hidden):
         raise KernelError(f"embedding output is {tuple(out.shape)}, expected {(n, hidden)}")
     _check("elementwise", library("elementwise").rocml_embed_gather(
-        _ptr(table), _code(table), _ptr(ids), _ptr(out), n, hidden, vocab, scale, _stream()))
+        _ptr(table), _code(table), _ptr(ids), _ptr(out), n, hidden, vocab, scale, _ptr(pos_table), _ptr(positions), max_pos,
+        _stream()))
 
 
 def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
@@ -198,12 +223,16 @@ def rmsnorm(x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
         stride, _stream()))
 
 
-GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2, "sigmoid_1702": 3}      # sigmoid_1702: g * sigmoid(1.702 g)
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool = False, activation: str = "silu") -> None:
-    """``out = act(gate) * up``.  ``gate_up`` rows hold the gate half then the up half, or (gate, up)
-    pairs when ``interleaved``; ``activation`` is one of ``GATE_ACTIVATIONS``."""
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool = False, activation: str = "silu",
+           limit: Optional[float] = None, up_offset: float = 0.0) -> None:
+    """``out = act(gate) * (up + up_offset)``.  ``gate_up`` rows hold the gate half then the up half, or
+    (gate, up) pairs when ``interleaved``; ``activation`` is one of ``GATE_ACTIVATIONS``.  ``limit``:
+    the gate is cut off above at ``limit`` and the up value is held inside ``[-limit, limit]`` first."""
+    if limit is not None and not limit > 0:
+        raise KernelError(f"the limit of a gated activation must be positive, got {limit}")
     if activation not in GATE_ACTIVATIONS:
         raise KernelError(f"unknown activation {activation!r}; known: {sorted(GATE_ACTIVATIONS)}")
     _dev(gate_up, out)
@@ -212,7 +241,7 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor, interleaved: bool = False, 
         raise KernelError(f"gate/up is {tuple(gate_up.shape)}, expected {(n_tokens, 2 * inter)}")
     _check("elementwise", library("elementwise").rocml_swiglu(
         _ptr(gate_up), _code(gate_up), _ptr(out), _code(out), n_tokens, inter, 1 if interleaved else 0,
-        GATE_ACTIVATIONS[activation], _stream()))
+        GATE_ACTIVATIONS[activation], 0.0 if limit is None else float(limit), float(up_offset), _stream()))
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
@@ -238,7 +267,7 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
                         v_cache: Optional[torch.Tensor], block_table: Optional[torch.Tensor],
                         token_seq: torch.Tensor, token_pos: torch.Tensor, write_kv: bool = True,
                         n_splits: int = 1, pairing: str = "halves", bias: Optional[torch.Tensor] = None,
-                        v_head_dim: Optional[int] = None) -> None:
+                        v_head_dim: Optional[int] = None, q_temp=None) -> None:
     """``qkv`` is ``[T, ld]`` with q, k, v side by side (k and v may be absent when
     ``write_kv`` is false).  Keys are ``[pages, Hkv, page_size, D]``, values
     ``[pages, Hkv, D, page_size]``.  ``pairing``: which two values of the rotated width turn
@@ -247,7 +276,11 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
     and appended (the caller's attention kernel prepares its queries itself).  ``bias``: 32-bit,
     one number per column of ``qkv``, added to the projection's sums.  ``v_head_dim``: the size of a
     value head when it is not ``head_dim`` (the value columns then follow the ``Hq + Hkv`` heads of
-    ``head_dim``)."""
+    ``head_dim``).  ``q_temp``: ``(coef, every)``; the query at position ``p`` is multiplied by
+    ``1 + coef * ln(floor((p + 1) / every) + 1)`` after its norm."""
+    qt_coef, qt_every = (0.0, 0) if q_temp is None else (float(q_temp[0]), int(q_temp[1]))
+    if q_temp is not None and qt_every <= 0:
+        raise KernelError(f"the period of the query's stretch must be positive, got {qt_every}")
     dv = head_dim if v_head_dim is None else int(v_head_dim)
     if pairing not in ROPE_PAIRINGS:
         raise KernelError(f"unknown rotation pairing {pairing!r}; known: {sorted(ROPE_PAIRINGS)}")
@@ -291,7 +324,8 @@ def qk_norm_rope_append(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_d
         _ptr(qkv), _code(qkv), ld, n_tokens, n_heads, n_kv_heads, head_dim, _ptr(q_gain), _ptr(k_gain),
         eps, _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, ROPE_PAIRINGS[pairing], _ptr(q_out), _ptr(k_cache),
         _ptr(v_cache), _code(q_out if q_out is not None else k_cache), _ptr(block_table), bt_width, _ptr(token_seq),
-        _ptr(token_pos), page_size, 1 if write_kv else 0, n_splits, split_stride, _ptr(bias), dv, _stream()))
+        _ptr(token_pos), page_size, 1 if write_kv else 0, n_splits, split_stride, _ptr(bias), dv, qt_coef, qt_every,
+        _stream()))
 
 
 def add_row_vector(x: torch.Tensor, b: torch.Tensor) -> None:
@@ -420,6 +454,42 @@ def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> None:
     ldg = gate.stride(0) if y.shape[0] > 1 else max(gate.stride(0), y.shape[1])
     _check("elementwise", library("elementwise").rocml_sigmoid_gate(_ptr(y), _code(y), _ptr(gate), ldg, y.shape[0],
                                                                    y.shape[1], _stream()))
+
+
+def sum_norm(x: torch.Tensor, branches: Sequence[torch.Tensor], branch_gains: Sequence[Optional[torch.Tensor]],
+             gain: Optional[torch.Tensor], eps: float, alpha: float = 1.0, weight: float = 1.0,
+             copy: Optional[torch.Tensor] = None) -> None:
+    """``x <- rms(alpha * x + weight * sum_b f_b(y_b)) * gain`` in place (32-bit; without ``gain`` the
+    sum itself, and with ``alpha`` zero ``x`` is only written), where
+    ``f_b(y) = rms(y) * gain_b`` for a branch with a gain and ``y`` itself for one without;
+    ``rms(v) = v / sqrt(mean(v^2) + eps)``.  ``copy`` gets the new ``x`` in its own type."""
+    _dev(x, gain, copy, *branches, *[g for g in branch_gains if g is not None])
+    _want(x, torch.float32, "residual stream")
+    if gain is not None:
+        _want(gain, torch.float32, "norm gain")
+    rows, n = x.shape
+    if not 1 <= len(branches) <= 4 or len(branch_gains) != len(branches):
+        raise KernelError("sum_norm takes one to four branches and a gain (or None) for each")
+    for y, g in zip(branches, branch_gains):
+        _want(y, torch.float32, "a branch's output")
+        if y.shape != x.shape or (g is not None and (g.dtype != torch.float32 or g.numel() != n)):
+            raise KernelError(f"a branch is {tuple(y.shape)} for a stream of {tuple(x.shape)}, or its gain does not fit")
+    if (gain is not None and gain.numel() != n) or (copy is not None and copy.shape != x.shape):
+        raise KernelError("sum_norm: gain or copy do not fit the stream")
+    ys = (ctypes.c_void_p * len(branches))(*[y.data_ptr() for y in branches])
+    gs = (ctypes.c_void_p * len(branches))(*[None if g is None else g.data_ptr() for g in branch_gains])
+    _check("elementwise", library("elementwise").rocml_sum_norm(
+        _ptr(x), rows, n, float(alpha), float(weight), len(branches), ys, gs, _ptr(gain), float(eps), _ptr(copy),
+        _code(copy) if copy is not None else 0, _stream()))
+
+
+def convert(x: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = x`` in ``out``'s type, for 32-bit ``x``."""
+    _dev(x, out)
+    _want(x, torch.float32, "the values to copy")
+    if x.numel() != out.numel():
+        raise KernelError("convert: sizes differ")
+    _check("elementwise", library("elementwise").rocml_convert(_ptr(x), _ptr(out), _code(out), x.numel(), _stream()))
 
 
 def add_into(x: torch.Tensor, y: torch.Tensor) -> None:
@@ -859,3 +929,152 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
         _ptr(logits), _ptr(work), batch, vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform),
         _ptr(penalty), _ptr(history), 0 if history is None else history.shape[1], _ptr(history_len),
         int(small_k), _ptr(out), _stream()))
+
+
+# ---- recurrent ---------------------------------------------------------------------------
+def causal_conv(u: torch.Tensor, col0: int, n_channels: int, w: torch.Tensor, bias: Optional[torch.Tensor],
+                state: torch.Tensor, token_seq: torch.Tensor, cu_seqlens: torch.Tensor, seq_slots: torch.Tensor,
+                out: torch.Tensor, silu: bool = True) -> None:
+    """Causal convolution per channel over columns ``col0 .. col0 + n_channels - 1`` of the 32-bit
+    ``u [T, ld]``: ``out[t, c] = act(bias[c] + sum_j w[c, j] in(t - (taps - 1) + j, c))``.  ``state``
+    ``[slots, taps - 1, channels]`` holds every sequence's last ``taps - 1`` inputs (zeros at its
+    start), is read for the inputs before the step's first token and brought up to date."""
+    _dev(u, w, bias, state, token_seq, cu_seqlens, seq_slots, out)
+    for t, what in ((u, "convolution input"), (w, "convolution weights"), (state, "convolution state"), (out, "convolution output")):
+        _want(t, torch.float32, what)
+    n_tokens, ld = u.shape
+    taps = w.shape[1]
+    n_seqs = seq_slots.numel()
+    if w.shape != (n_channels, taps) or (bias is not None and (bias.dtype != torch.float32 or bias.numel() != n_channels)):
+        raise KernelError(f"convolution weights {tuple(w.shape)} or bias do not fit {n_channels} channels")
+    if out.shape != (n_tokens, n_channels) or token_seq.numel() != n_tokens or cu_seqlens.numel() != n_seqs + 1:
+        raise KernelError("convolution output or token tables do not fit the step")
+    if state.dim() != 3 or state.shape[1:] != (max(taps - 1, 0), n_channels):
+        raise KernelError(f"convolution state {tuple(state.shape)} does not fit {taps} taps of {n_channels} channels")
+    _check("recurrent", library("recurrent").rocml_causal_conv(
+        _ptr(u), ld, col0, n_tokens, n_channels, taps, _ptr(w), _ptr(bias), _ptr(state), state.shape[0], _ptr(token_seq),
+        _ptr(cu_seqlens), _ptr(seq_slots), n_seqs, _ptr(out), 1 if silu else 0, _stream()))
+
+
+def ssd_scan(xbc: torch.Tensor, dt_src: torch.Tensor, dt_col0: int, dt_bias: torch.Tensor, a_log: torch.Tensor,
+             d_skip: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor, seq_slots: torch.Tensor, y: torch.Tensor,
+             n_heads: int, head_dim: int, n_state: int, n_groups: int) -> None:
+    """The recurrence with a scalar decay per head over the step's tokens, per sequence in order:
+    ``dt = softplus(raw + dt_bias)``, ``S <- exp(-exp(A_log) dt) S + dt B x^T``, ``y = S^T C + D x``.
+    ``xbc [T, H P + 2 G N]`` holds x, B and C side by side, the raw step sizes are columns
+    ``dt_col0 .. dt_col0 + H - 1`` of ``dt_src``; ``state [slots, H, P, N]``; all 32-bit."""
+    _dev(xbc, dt_src, dt_bias, a_log, d_skip, state, cu_seqlens, seq_slots, y)
+    for t, what in ((xbc, "recurrence inputs"), (dt_src, "step sizes"), (dt_bias, "dt_bias"), (a_log, "A_log"),
+                    (d_skip, "D"), (state, "recurrent state"), (y, "recurrence output")):
+        _want(t, torch.float32, what)
+    n_tokens = xbc.shape[0]
+    n_seqs = seq_slots.numel()
+    if state.dim() != 4 or state.shape[1:] != (n_heads, head_dim, n_state):
+        raise KernelError(f"recurrent state {tuple(state.shape)} does not fit {n_heads} heads of {head_dim} x {n_state}")
+    if y.shape != (n_tokens, n_heads * head_dim) or dt_src.shape[0] != n_tokens or cu_seqlens.numel() != n_seqs + 1:
+        raise KernelError("recurrence output or tables do not fit the step")
+    if min(dt_bias.numel(), a_log.numel(), d_skip.numel()) != n_heads or max(dt_bias.numel(), a_log.numel(), d_skip.numel()) != n_heads:
+        raise KernelError("dt_bias, A_log and D must have one number per head")
+    _check("recurrent", library("recurrent").rocml_ssd_scan(
+        _ptr(xbc), xbc.shape[1], _ptr(dt_src), dt_src.shape[1], dt_col0, _ptr(dt_bias), _ptr(a_log), _ptr(d_skip),
+        _ptr(state), state.shape[0], _ptr(cu_seqlens), _ptr(seq_slots), n_seqs, n_tokens, _ptr(y), n_heads, head_dim,
+        n_state, n_groups, _stream()))
+
+
+def gated_part_norm(y: torch.Tensor, z: torch.Tensor, z_col0: int, gain: torch.Tensor, out: torch.Tensor, parts: int,
+                    eps: float) -> None:
+    """``out = rms_parts(y * silu(z)) * gain``: the gate first, then each of the ``parts`` equal parts
+    of a row divided by its own root mean square.  ``z`` is columns ``z_col0 ..`` of a 32-bit matrix."""
+    _dev(y, z, gain, out)
+    for t, what in ((y, "norm input"), (z, "gate"), (gain, "norm gain")):
+        _want(t, torch.float32, what)
+    rows, n = y.shape
+    if gain.numel() != n or out.shape != y.shape or z.shape[0] != rows:
+        raise KernelError("gated_part_norm: sizes differ")
+    _check("recurrent", library("recurrent").rocml_gated_part_norm(
+        _ptr(y), _ptr(z), z.shape[1], z_col0, _ptr(gain), _ptr(out), _code(out), rows, n, parts, float(eps), _stream()))
+
+
+# ---- experts -----------------------------------------------------------------------------
+MOE_TILE_ROWS = 64
+
+
+def moe_max_tiles(n_pairs: int, n_experts: int) -> int:
+    """Room for the tiles of a plan: an expert's last tile may be short."""
+    return max(1, min(n_pairs, n_pairs // MOE_TILE_ROWS + n_experts))
+
+
+def moe_route(logits: torch.Tensor, top: int, groups, sum_eps: float, chosen: torch.Tensor, weight: torch.Tensor) -> None:
+    """Softmax over all experts, the ``top`` best (of the experts of the ``groups[1]`` best of
+    ``groups[0]`` equal groups of neighbours, a group's score being its largest, if ``groups`` is
+    given), weights = chosen scores / (their sum + ``sum_eps``).  ``chosen`` int32, ``weight`` float32,
+    both ``[T, top]``."""
+    _dev(logits, chosen, weight)
+    _want(logits, torch.float32, "router logits")
+    _want(chosen, torch.int32, "chosen experts")
+    _want(weight, torch.float32, "expert weights")
+    n_tokens, n_experts = logits.shape
+    if chosen.shape != (n_tokens, top) or weight.shape != (n_tokens, top):
+        raise KernelError("moe_route: outputs must be [tokens, top]")
+    count, keep = (0, 0) if groups is None else (int(groups[0]), int(groups[1]))
+    _check("moe", library("moe").rocml_moe_route(_ptr(logits), n_tokens, n_experts, top, count, keep, float(sum_eps),
+                                                 _ptr(chosen), _ptr(weight), _stream()))
+
+
+def moe_plan(chosen: torch.Tensor, n_experts: int, plan: torch.Tensor):
+    """Sorts the (token, choice) pairs by expert.  ``plan`` is int32 scratch of at least
+    ``moe_plan_words(pairs, experts)`` words; returns its views
+    ``(offsets [E + 1], order [pairs], place [pairs], tiles [2 * max_tiles], n_tiles [1], max_tiles)``."""
+    _dev(chosen, plan)
+    _want(chosen, torch.int32, "chosen experts")
+    _want(plan, torch.int32, "plan")
+    n_pairs = chosen.numel()
+    max_tiles = moe_max_tiles(n_pairs, n_experts)
+    if plan.numel() < moe_plan_words(n_pairs, n_experts):
+        raise KernelError("moe_plan: the plan's scratch is too small")
+    at = 0
+    views = []
+    for n in (n_experts + 1, n_pairs, n_pairs, 2 * max_tiles, 1):
+        views.append(plan[at:at + n])
+        at += n
+    offsets, order, place, tiles, n_tiles = views
+    _check("moe", library("moe").rocml_moe_plan(_ptr(chosen), n_pairs, n_experts, _ptr(offsets), _ptr(order), _ptr(place),
+                                                _ptr(tiles), _ptr(n_tiles), max_tiles, _stream()))
+    return offsets, order, place, tiles, n_tiles, max_tiles
+
+
+def moe_plan_words(n_pairs: int, n_experts: int) -> int:
+    return n_experts + 1 + 2 * n_pairs + 2 * moe_max_tiles(n_pairs, n_experts) + 1
+
+
+def moe_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, plan, top: int, gather: bool,
+             w2: Optional[torch.Tensor] = None, plain: bool = False) -> None:
+    """The products of all experts over the plan's order: row ``r`` of ``out`` (a place of expert
+    ``e``) is ``w[e] @ a_r``, with ``a_r`` the row of the pair's token when ``gather`` (``a`` holds the
+    step's tokens) and row ``r`` of ``a`` otherwise.  With ``w2``: ``silu(w[e] a_r) * (w2[e] a_r)``.
+    ``w`` is ``[experts, n, k]``."""
+    offsets, order, place, tiles, n_tiles, max_tiles = plan
+    _dev(a, w, w2, out)
+    n_experts, n, k = w.shape
+    if w2 is not None and (w2.shape != w.shape or w2.dtype != w.dtype):
+        raise KernelError("moe_gemm: the second matrix must have the first one's shape and type")
+    n_pairs = order.numel()
+    if a.shape[1] != k or out.shape != (n_pairs, n) or a.dtype != w.dtype:
+        raise KernelError(f"moe_gemm: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit {n_pairs} pairs")
+    _check("moe", library("moe").rocml_moe_gemm(
+        _ptr(a), _code(a), a.shape[1], a.shape[0], _ptr(order) if gather else None, top, _ptr(w), _ptr(w2), _code(w), n * k, k,
+        n_experts, _ptr(out), _code(out), n, n_pairs, n, k, _ptr(offsets), _ptr(tiles), _ptr(n_tiles), max_tiles,
+        1 if plain else 0, _stream()))
+
+
+def moe_combine(y: torch.Tensor, plan, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """``out[t] (+)= sum_c weight[t, c] * y[place[t * top + c]]`` (32-bit, choices in order)."""
+    offsets, order, place, tiles, n_tiles, max_tiles = plan
+    _dev(y, weight, out)
+    for t, what in ((y, "expert outputs"), (weight, "expert weights"), (out, "feed-forward output")):
+        _want(t, torch.float32, what)
+    n_tokens, top = weight.shape
+    if y.shape != (n_tokens * top, out.shape[1]) or out.shape[0] != n_tokens:
+        raise KernelError("moe_combine: sizes differ")
+    _check("moe", library("moe").rocml_moe_combine(_ptr(y), _ptr(place), _ptr(weight), _ptr(out), n_tokens, top, out.shape[1],
+                                                   1 if accumulate else 0, _stream()))

@@ -50,6 +50,12 @@ class Attention(Mixer):
         # what the matrix-core kernels do not know: such a layer runs the plain attention kernel
         self.extras = (self.v_head_dim != spec.head_dim or spec.chunk is not None
                        or spec.distance_slopes is not None or spec.sink)
+        if spec.q_temp is not None and not (spec.q_temp[1] > 0):
+            raise ConfigError(f"the period of the query's stretch must be positive, got {spec.q_temp[1]}")
+        # what only the norm-and-rotation kernel knows (the kernels that prepare their queries
+        # themselves do not): a stretch of the query with its position, an output gate
+        self.separate_q = spec.q_temp is not None or spec.gate
+        self.norm_learned = spec.qk_norm is None or getattr(spec.qk_norm, "learned", True)
         self.slopes: Optional[torch.Tensor] = None
         if spec.distance_slopes is not None and torch.device(ctx.device).type != "meta":
             self.slopes = torch.tensor(spec.distance_slopes, dtype=torch.float32, device=ctx.device)
@@ -60,6 +66,7 @@ class Attention(Mixer):
         self.kv_dim = spec.n_kv_heads * spec.head_dim
         self.v_dim = spec.n_kv_heads * self.v_head_dim
         self.o_dim = spec.n_heads * self.v_head_dim
+        self.g_dim = self.o_dim if spec.gate else 0
         self.position = build_position(spec.position, ctx) if spec.position is not None else None
         self.pairing = getattr(self.position, "pairing", "halves")
         if self.pairing not in ops.ROPE_PAIRINGS:
@@ -86,23 +93,29 @@ class Attention(Mixer):
                           "k_proj.bias": ParamSpec((self.kv_dim,), role="gain", init="normal"),
                           "v_proj.bias": ParamSpec((self.v_dim,), role="gain", init="normal"),
                           "o_proj.bias": ParamSpec((s.hidden,), role="gain", init="normal")})
-        if s.qk_norm is not None:
+        if s.qk_norm is not None and self.norm_learned:
             specs["q_norm.weight"] = ParamSpec((s.head_dim,), role="gain", init="gain")
             specs["k_norm.weight"] = ParamSpec((s.head_dim,), role="gain", init="gain")
+        if s.gate:
+            specs["g_proj.weight"] = ParamSpec((self.g_dim, s.hidden))
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         # One [Q + 2 KV, hidden] matrix: q rows first, so a layer that only reads another
         # layer's cache multiplies by the leading Q rows.
-        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
-                                tensors["v_proj.weight"]], dim=0).contiguous()
+        # (an output gate's rows come last: its projection rides in the same product)
+        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+                               + ([tensors["g_proj.weight"]] if self.spec.gate else []), dim=0).contiguous()
         self.w_o = tensors["o_proj.weight"]
         if self.spec.bias:
             self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]).contiguous()
             self.b_o = tensors["o_proj.bias"]
         if self.spec.qk_norm is not None:
-            self.q_gain = tensors["q_norm.weight"]
-            self.k_gain = tensors["k_norm.weight"]
+            if self.norm_learned:
+                self.q_gain = tensors["q_norm.weight"]
+                self.k_gain = tensors["k_norm.weight"]
+            else:       # a norm without a weight: the kernels take a gain of ones
+                self.q_gain = self.k_gain = torch.ones(self.spec.head_dim, dtype=torch.float32, device=self.w_o.device)
 
     def flops(self, new_counts, starts) -> int:
         # the products with the weights, and 4 * heads * head size per query and key it sees
@@ -126,7 +139,7 @@ class Attention(Mixer):
     def _fused_decode(self, step) -> bool:
         rot = None if self.position is None else self.position.rot_dim
         # (blocks, slopes, a sink and biases ride in the fused kernel; a value head of another size does not)
-        return self.v_head_dim == self.spec.head_dim and step.max_new == 1 and ops.attention_decode_fusable(
+        return not self.separate_q and self.v_head_dim == self.spec.head_dim and step.max_new == 1 and ops.attention_decode_fusable(
             self.dtype, self.spec.n_heads, self.spec.n_kv_heads, self.spec.head_dim, ops.FUSED_DECODE_PAGE, rot, self.pairing)
 
     def _fused_prefill(self, step, cache) -> bool:
@@ -134,7 +147,7 @@ class Attention(Mixer):
         tokens on (the preparation lengthens every attention block by some 6 us, the norm-and-rotation
         kernel's q rows cost 8 us per thousand tokens at 32 heads of 128)."""
         rot = None if self.position is None else self.position.rot_dim
-        return (not self.extras and not self.spec.bias and step.max_new > 1 and step.n_tokens >= self.FUSED_PREFILL_MIN_TOKENS
+        return (not self.extras and not self.separate_q and not self.spec.bias and step.max_new > 1 and step.n_tokens >= self.FUSED_PREFILL_MIN_TOKENS
                 and step.cu_seqlens is not None and self.dtype == torch.bfloat16
                 and ops.attention_prefill_fusable(cache.k.dtype, self.spec.head_dim, cache.k.shape[2], rot, self.pairing))
 
@@ -160,12 +173,15 @@ class Attention(Mixer):
         s = self.spec
         n = step.n_tokens
         ws = step.workspace
-        rows = self.q_dim + self.kv_dim + self.v_dim if owns_cache else self.q_dim
+        rows = self.q_dim + self.kv_dim + self.v_dim + self.g_dim if owns_cache else self.q_dim
+        if s.gate and not owns_cache:
+            raise ConfigError("a gated attention layer that reads another layer's cache is not supported")
         qkv = ws.get("attn.qkv", (n, rows), torch.float32)
         scratch = ws.scratch()
         # (the decode kernel that reads the projection adds four partial sums in one trip to memory
         # and further ones one after the other: K is cut into few pieces for it)
-        splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=True,
+        # (the gate's columns are read where they lie: the product is then completed)
+        splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=not s.gate,
                           max_splits=ops.FUSED_DECODE_SPLITS if self._fused_decode(step) else 0)
         if splits:      # the product's split-K partial sums; the next kernel adds them
             qkv = scratch[:splits * n * rows * 4].view(torch.float32).view(splits, n, rows)
@@ -207,12 +223,14 @@ class Attention(Mixer):
                 ops.qk_norm_rope_append(qkv, s.n_heads, s.n_kv_heads, s.head_dim, self.q_gain, self.k_gain, eps,
                                         cos, sin, rot, q, cache.k, cache.v, cache.block_table, step.token_seq,
                                         step.token_pos, write_kv=owns_cache, n_splits=max(splits, 1), pairing=self.pairing,
-                                        bias=bias, v_head_dim=self.v_head_dim)
+                                        bias=bias, v_head_dim=self.v_head_dim, q_temp=s.q_temp)
                 ops.attention(q, o, cache.k, cache.v, cache.block_table, step.token_seq, step.token_pos,
                               s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, workspace=ws.scratch(),
                               cu_seqlens=step.cu_seqlens, max_new=step.max_new, q_counts=step.new_counts,
                               max_len=step.max_len, n_splits=self._decode_splits(step, cache),
                               v_head_dim=self.v_head_dim, chunk=s.chunk, slopes=self.slopes, sink=s.sink)
+        if s.gate:
+            ops.sigmoid_gate(o, qkv[:, rows - self.g_dim:])
         if self.b_o is not None:
             ws.flush_pending()
             ops.add_row_vector(x_accum, self.b_o)

@@ -81,6 +81,14 @@ class StateRequest:
     dtype: torch.dtype = torch.float32
 
 
+@dataclass(frozen=True)
+class CompositeRequest:
+    """What a mixer made of several parts asks for: one request per part (None for a part that
+    keeps nothing; a part's request may be composite again).  Every part gets storage of its own
+    and the mixer sees them as ``view.parts``, in this order."""
+    parts: Tuple[Optional[Any], ...]
+
+
 class Part:
     # False: forward() waits for the GPU or works on the host (reads a tensor back, loops over
     # tokens), so a decode step with this part cannot be recorded and replayed as a graph

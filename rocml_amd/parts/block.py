@@ -2,14 +2,20 @@
 
 ``pre_norm`` is the reference's wiring (rocml/src/forward/chunk_forward.rs:107-135):
 ``x += mixer(norm(x))``, then ``x += ffn(norm(x))``; the residual stream ``x`` stays
-32-bit and the normalised copy has the activation type."""
+32-bit and the normalised copy has the activation type.
+
+``post_norm`` norms after the sum: ``x <- norm(a x + mixer(x))``, then ``x <- norm(a x + ffn(x))`` with
+``a`` the block's ``residual_scale``; the sublayers read the stream itself."""
 from __future__ import annotations
 
 from typing import Dict
 
+from .. import ops
+
 import torch
 
 from ..config.spec import BlockSpec
+from ..errors import ConfigError
 from .base import BuildContext, ParamSpec, Part
 from .registry import build_feed_forward, build_mixer, build_norm, register_block
 from .residual import stream
@@ -109,3 +115,96 @@ class PreNormBlock(Part):
 
 
 register_block("pre_norm", PreNormBlock)
+
+_COPY_KEY = "post_norm.stream_copy"
+
+
+class PostNormBlock(Part):
+    """``x <- norm1(a x + mixer(x))``, ``x <- norm2(a x + ffn(x))``.  A sublayer reads the stream itself
+    (in the compute type: a copy that the norm kernel before it wrote, the stream itself in 32-bit)
+    and writes its result to a buffer of the block; one kernel then forms the scaled residual sum and
+    its norm in 32-bit, in place, and the copy for the next sublayer.  A mixer that is a sum of normed
+    branches hands its branches over as they are (``branches``) and the same kernel norms and sums
+    them on the way."""
+    takes_pending = False
+    takes_next_norm = False
+
+    def __init__(self, spec: BlockSpec, ctx: BuildContext):
+        self.dtype = ctx.dtype
+        self.hidden = spec.mixer_norm.size
+        self.alpha = float(spec.residual_scale)
+        self.children = {"mixer_norm": build_norm(spec.mixer_norm, ctx),
+                         "mixer": build_mixer(spec.mixer, ctx)}
+        if spec.ffn is not None:
+            self.children["ffn_norm"] = build_norm(spec.ffn_norm, ctx)
+            self.children["ffn"] = build_feed_forward(spec.ffn, ctx)
+        self.mixer_norm = self.children["mixer_norm"]
+        self.mixer = self.children["mixer"]
+        self.ffn_norm = self.children.get("ffn_norm")
+        self.ffn = self.children.get("ffn")
+        for norm in (self.mixer_norm, self.ffn_norm):
+            if norm is not None and (not hasattr(norm, "gain") or not hasattr(norm, "eps")):
+                raise ConfigError("a block that norms after the sum needs norms of the root-mean-square kind")
+        self.graph_safe = all(getattr(c, "graph_safe", True) for c in self.children.values())
+        self.prompt_graph_safe = all(getattr(c, "prompt_graph_safe", False) for c in self.children.values())
+        self.kernel_families = tuple(f for c in self.children.values() for f in getattr(c, "kernel_families", ()))
+
+    param_specs = PreNormBlock.param_specs
+    bind = PreNormBlock.bind
+    cache_request = PreNormBlock.cache_request
+    flops = PreNormBlock.flops
+
+    def activation_bytes(self, n_tokens: int) -> int:
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        return n_tokens * self.hidden * (size + 4) + self.mixer.activation_bytes(n_tokens) + \
+            (self.ffn.activation_bytes(n_tokens) if self.ffn is not None else 0)
+
+    def _operand(self, step, x: torch.Tensor) -> torch.Tensor:
+        """The stream as the products' operand."""
+        if self.dtype == torch.float32:
+            return x
+        found = step.memo.get(_COPY_KEY)
+        if found is not None and found[0] == x.data_ptr():
+            return found[1]
+        xb = step.workspace.get("block.stream_copy", tuple(x.shape), self.dtype)
+        ops.convert(x, xb)
+        step.memo[_COPY_KEY] = (x.data_ptr(), xb)
+        return xb
+
+    def _sum_norm(self, step, x, outs, gains, weight, norm) -> None:
+        copy = None
+        if self.dtype != torch.float32:
+            copy = step.workspace.get("block.stream_copy", tuple(x.shape), self.dtype)
+        ops.sum_norm(x, outs, gains, norm.gain, norm.eps, alpha=self.alpha, weight=weight, copy=copy)
+        if copy is not None:
+            step.memo[_COPY_KEY] = (x.data_ptr(), copy)
+
+    def forward(self, step, x: torch.Tensor, cache, owns_cache: bool) -> None:
+        ws = step.workspace
+        rs = stream(step)
+        ws.flush_pending()
+        rs.row_scale = rs.next_norm = None
+        xb = self._operand(step, x)
+        rs.overwrite = True
+        try:
+            if hasattr(self.mixer, "branches"):
+                outs, gains, weight = self.mixer.branches(step, xb, cache, owns_cache)
+            else:
+                y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
+                self.mixer.forward(step, xb, y, cache, owns_cache)
+                outs, gains, weight = [y], [None], 1.0
+            ws.flush_pending()
+            self._sum_norm(step, x, outs, gains, weight, self.mixer_norm)
+            if self.ffn is None:
+                return
+            xb = self._operand(step, x)
+            y = ws.get("block.sublayer", tuple(x.shape), torch.float32)
+            rs.overwrite = True
+            self.ffn.forward(step, xb, y)
+            ws.flush_pending()
+            self._sum_norm(step, x, [y], [None], 1.0, self.ffn_norm)
+        finally:
+            rs.overwrite = False
+
+
+register_block("post_norm", PostNormBlock)

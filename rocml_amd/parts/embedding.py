@@ -7,7 +7,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from ..config.spec import TokenTableSpec
+from ..config.spec import TokenPositionTableSpec, TokenTableSpec
 from .base import BuildContext, Embedding, ParamSpec
 from .registry import register_embedding
 
@@ -35,3 +35,33 @@ class TokenTable(Embedding):
 
 
 register_embedding("token_table", TokenTable)
+
+
+class TokenPositionTable(Embedding):
+    """A token's row times ``scale`` plus the learned row of its position (not scaled), in 32-bit."""
+    prompt_graph_safe = True
+
+    def __init__(self, spec: TokenPositionTableSpec, ctx: BuildContext):
+        self.vocab = spec.vocab
+        self.hidden = spec.hidden
+        self.max_positions = spec.max_positions
+        self.scale = float(spec.scale)
+        self.table: Optional[torch.Tensor] = None
+        self.positions: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.vocab, self.hidden)),
+                "positions": ParamSpec((self.max_positions, self.hidden))}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.table = tensors["weight"]
+        self.positions = tensors["positions"]
+
+    def shared_matrix(self) -> Optional[torch.Tensor]:
+        return self.table
+
+    def forward(self, step, x: torch.Tensor) -> None:
+        ops.embed_gather(self.table, step.token_ids, x, self.scale, pos_table=self.positions, positions=step.token_pos)
+
+
+register_embedding("token_position_table", TokenPositionTable)

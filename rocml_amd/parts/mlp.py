@@ -2,7 +2,8 @@
 (rocml/src/forward/ffn.rs:36-107, rocml-kernels/kernels/silu_mul.hip:12-20).  Gate and up
 are one product over the concatenated weight; the residual sum is the down product's
 epilogue.  ``act`` is the spec's: ``silu`` and ``relu`` are epilogues of the gate/up product,
-``gelu_tanh`` runs as a kernel of its own behind it."""
+``gelu_tanh`` and ``sigmoid_1702`` (``g sigmoid(1.702 g)``) run as a kernel of their own behind it, and so
+does any layer with a ``limit`` on gate and up values or an offset added to the up values."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -26,6 +27,12 @@ class GatedMlp(FeedForward):
             raise ConfigError(f"activation {spec.activation!r} is not supported; known: {sorted(ops.GATE_ACTIVATIONS)}")
         # the product's epilogue for this activation, if it has one
         self.epilogue = {"silu": "swiglu", "relu": "relu_glu"}.get(spec.activation)
+        self.limit = getattr(spec, "limit", None)
+        self.up_offset = float(getattr(spec, "up_offset", 0.0))
+        if self.limit is not None and not self.limit > 0:
+            raise ConfigError(f"the limit of the gated activation must be positive, got {self.limit}")
+        if self.limit is not None or self.up_offset != 0.0:
+            self.epilogue = None          # the products' epilogues know the bare activations only
         self.spec = spec
         self.dtype = ctx.dtype
         self.w_gate_up: Optional[torch.Tensor] = None
@@ -67,7 +74,7 @@ class GatedMlp(FeedForward):
                 raise ConfigError("the feed-forward was handed an input without its norm's scale in a step it cannot scale")
             gate_up = ws.get("mlp.gate_up", (n, 2 * s.intermediate), torch.float32)
             ops.gemm(xn, self.w_gate_up, gate_up, workspace=ws.scratch())
-            ops.swiglu(gate_up, h, interleaved=True, activation=s.activation)
+            ops.swiglu(gate_up, h, interleaved=True, activation=s.activation, limit=self.limit, up_offset=self.up_offset)
         stream(step).add_product(h, self.w_down, x_accum)
 
 

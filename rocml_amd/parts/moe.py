@@ -1,0 +1,93 @@
+"""A feed-forward of many small gated feed-forwards (experts) of which each token uses a few.
+
+The router's logits are a product with 32-bit sums, the scores (softmax over all experts), the
+choice (the best experts, optionally only of the best groups of neighbouring experts) and the
+weights (chosen scores over their sum) are 32-bit.  The step's (token, choice) pairs are sorted by
+expert on the device, all experts' first two products and their activation run as one launch over
+the sorted rows, the down products as a second, and the weighted sum of a token's experts is
+32-bit, in the order of the choices.  Nothing is read back to the host, so a step can be recorded.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from ..config.spec import RoutedExpertsSpec
+from ..errors import ConfigError
+from .base import BuildContext, FeedForward, ParamSpec
+from .registry import register_feed_forward
+from .residual import stream
+
+
+class RoutedExperts(FeedForward):
+    adds_only = True
+    prompt_graph_safe = True
+    kernel_families = ("moe",)
+
+    def __init__(self, spec: RoutedExpertsSpec, ctx: BuildContext):
+        if spec.activation != "silu":
+            raise ConfigError(f"the experts' activation {spec.activation!r} is not supported; known: silu")
+        if not 1 <= spec.top <= min(spec.n_experts, 64):
+            raise ConfigError(f"a token uses {spec.top} of {spec.n_experts} experts; at least 1 and at most 64")
+        if spec.n_experts > 512:
+            raise ConfigError(f"{spec.n_experts} experts exceed the 512 the routing kernel takes")
+        if spec.groups is not None:
+            count, keep = spec.groups
+            if count <= 0 or spec.n_experts % count != 0 or not 1 <= keep <= count or spec.top > keep * (spec.n_experts // count):
+                raise ConfigError(f"{spec.n_experts} experts in {count} groups of which {keep} are kept do not allow "
+                                  f"{spec.top} choices")
+        self.spec = spec
+        self.dtype = ctx.dtype
+        self.w_router: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        s = self.spec
+        specs = {"router.weight": ParamSpec((s.n_experts, s.hidden))}
+        for e in range(s.n_experts):
+            specs[f"experts.{e}.gate_proj.weight"] = ParamSpec((s.intermediate, s.hidden))
+            specs[f"experts.{e}.up_proj.weight"] = ParamSpec((s.intermediate, s.hidden))
+            specs[f"experts.{e}.down_proj.weight"] = ParamSpec((s.hidden, s.intermediate))
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        n = self.spec.n_experts
+        self.w_router = tensors["router.weight"]
+        # one tensor per kind, expert after expert: a launch reaches every expert's matrix by a stride
+        self.w_gate = torch.stack([tensors[f"experts.{e}.gate_proj.weight"] for e in range(n)]).contiguous()
+        self.w_up = torch.stack([tensors[f"experts.{e}.up_proj.weight"] for e in range(n)]).contiguous()
+        self.w_down = torch.stack([tensors[f"experts.{e}.down_proj.weight"] for e in range(n)]).contiguous()
+
+    def matrix_elements(self) -> int:
+        """What a token is multiplied with: the router and the experts it uses."""
+        s = self.spec
+        return s.n_experts * s.hidden + s.top * 3 * s.hidden * s.intermediate
+
+    def activation_bytes(self, n_tokens: int) -> int:
+        s = self.spec
+        size = 2 if self.dtype == torch.bfloat16 else 4
+        return n_tokens * (s.n_experts * 4 + s.top * (s.intermediate * size + s.hidden * 4 + 16))
+
+    def forward(self, step, xn, x_accum) -> None:
+        s = self.spec
+        n = step.n_tokens
+        ws = step.workspace
+        logits = ws.get("moe.logits", (n, s.n_experts), torch.float32)
+        ops.gemm(xn, self.w_router, logits, workspace=ws.scratch())
+        chosen = ws.get("moe.chosen", (n, s.top), torch.int32)
+        weight = ws.get("moe.weight", (n, s.top), torch.float32)
+        ops.moe_route(logits, s.top, s.groups, s.sum_eps, chosen, weight)
+        pairs = n * s.top
+        plan = ops.moe_plan(chosen, s.n_experts, ws.get("moe.plan", (ops.moe_plan_words(pairs, s.n_experts),), torch.int32))
+        h = ws.get("moe.h", (pairs, s.intermediate), self.dtype)
+        ops.moe_gemm(xn, self.w_gate, h, plan, s.top, gather=True, w2=self.w_up)
+        y = ws.get("moe.y", (pairs, s.hidden), torch.float32)
+        ops.moe_gemm(h, self.w_down, y, plan, s.top, gather=False)
+        accumulate = not stream(step).overwrite
+        if accumulate:
+            ws.flush_pending()        # the stream must be whole before this kernel adds to it
+        ops.moe_combine(y, plan, weight, x_accum, accumulate=accumulate)
+
+
+register_feed_forward("routed_experts", RoutedExperts)

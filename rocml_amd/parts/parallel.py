@@ -1,0 +1,88 @@
+"""A set of mixers that all run on one input: the result is ``weight * sum_b norm_b(out_b)``,
+every branch's output normed over the model width with a gain of its own.
+
+A branch is any registered mixer, built from its spec; each keeps what it needs in the cache
+through a part of a composite request.  The branches' outputs stay in buffers of their own: a block
+that norms after its sum takes them as they are (``branches``) and does the branches' norms, their
+sum, the residual sum and its own norm in one kernel; in any other block ``forward`` adds the
+weighted sum to the stream.
+"""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from .. import ops
+from ..config.spec import ParallelMixerSpec
+from ..errors import ConfigError
+from .base import BuildContext, CompositeRequest, Mixer, ParamSpec
+from .registry import build_mixer, register_mixer
+from .residual import stream
+
+
+class ParallelMixer(Mixer):
+    adds_only = True
+
+    def __init__(self, spec: ParallelMixerSpec, ctx: BuildContext):
+        if not 1 <= len(spec.branches) <= 4:
+            raise ConfigError(f"a parallel mixer has one to four branches, got {len(spec.branches)}")
+        names = [name for name, _ in spec.branches]
+        if len(set(names)) != len(names):
+            raise ConfigError(f"the branches of a parallel mixer need different names, got {names}")
+        self.spec = spec
+        self.dtype = ctx.dtype
+        self.children = {name: build_mixer(sub, ctx) for name, sub in spec.branches}
+        self.graph_safe = all(getattr(c, "graph_safe", True) for c in self.children.values())
+        self.prompt_graph_safe = all(getattr(c, "prompt_graph_safe", False) for c in self.children.values())
+        self.kernel_families = tuple(f for c in self.children.values() for f in getattr(c, "kernel_families", ()))
+        self.gains: Dict[str, torch.Tensor] = {}
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        specs = {}
+        for name, child in self.children.items():
+            for p, ps in child.param_specs().items():
+                specs[f"{name}.{p}"] = ps
+            specs[f"{name}.out_norm.weight"] = ParamSpec((self.spec.hidden,), role="gain", init="gain")
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for name, child in self.children.items():
+            prefix = name + "."
+            own = {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
+            self.gains[name] = own.pop("out_norm.weight")
+            child.bind(own)
+
+    def cache_request(self) -> CompositeRequest:
+        return CompositeRequest(tuple(child.cache_request() for child in self.children.values()))
+
+    def flops(self, new_counts, starts) -> int:
+        return sum(child.flops(new_counts, starts) for child in self.children.values())
+
+    def activation_bytes(self, n_tokens: int) -> int:
+        return sum(child.activation_bytes(n_tokens) + n_tokens * self.spec.hidden * 4 for child in self.children.values())
+
+    def branches(self, step, xn, cache, owns_cache: bool):
+        """Runs every branch on ``xn`` and returns ``(outputs, gains, weight)``: the mixer's result is
+        ``weight * sum_b rms(outputs[b]) * gains[b]``; the outputs are 32-bit ``[tokens, hidden]``."""
+        ws = step.workspace
+        rs = stream(step)
+        before = rs.overwrite
+        views = cache.parts if cache is not None else (None,) * len(self.children)
+        outs: List[torch.Tensor] = []
+        for i, (name, child) in enumerate(self.children.items()):
+            y = ws.get(f"parallel.y{i}", (step.n_tokens, self.spec.hidden), torch.float32)
+            rs.overwrite = True
+            child.forward(step, xn, y, views[i], owns_cache)
+            ws.flush_pending()
+            outs.append(y)
+        rs.overwrite = before
+        return outs, [self.gains[name] for name in self.children], float(self.spec.weight)
+
+    def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
+        outs, gains, weight = self.branches(step, xn, cache, owns_cache)
+        step.workspace.flush_pending()
+        ops.sum_norm(x_accum, outs, gains, None, self.spec.eps, alpha=0.0 if stream(step).overwrite else 1.0, weight=weight)
+
+
+register_mixer("parallel", ParallelMixer)

@@ -34,6 +34,9 @@ class ResidualStream:
         self.next_norm: Optional[NormHint] = None
         # set around a part's forward: its input lacks this scale (an ``ops.RowScale``)
         self.row_scale = None
+        # set around a part's forward by a block whose sublayers do not add to the stream: the part's
+        # target is a buffer of the block's, and the part's last product writes it instead of adding to it
+        self.overwrite = False
         self._prescaled = None
 
     def add_product(self, a: torch.Tensor, w: torch.Tensor, target: torch.Tensor) -> None:
@@ -42,6 +45,10 @@ class ResidualStream:
         ws = self.workspace
         hint = self.next_norm
         self._prescaled = None
+        if self.overwrite:
+            ws.flush_pending()
+            ops.gemm(a, w, target, accumulate=False, workspace=ws.scratch())
+            return
         if hint is not None and target.dtype == torch.float32 and hint.width == target.shape[1] \
                 and ops.gemm_residual_prescale_pays(a, w):
             ws.flush_pending()
