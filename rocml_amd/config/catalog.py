@@ -89,6 +89,31 @@ CATALOG += [
     ModelEntry("dokulix-2b", _dokulix(32768, 2048, 6144, 16, 8, 128, 768, 512, 64, 1024, 1024, 24)),
 ]
 
+
+
+def felovik_config(vocab, width, heads, kv_heads, dim, ssm_heads, ssm_dim, state, groups, ff, experts, expert_ff, top, n_layers,
+                   max_positions=8192, dense_every=4):
+    """A Felovik configuration: every layer the attention and the recurrence next to each other, a dense
+    feed-forward in every ``dense_every``-th layer (the first among them) and routed experts in the others."""
+    mixer = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                      "q_temp": {"coef": 0.1, "every": 1024}},
+             "right": {"heads": ssm_heads, "vdim": ssm_dim, "state": state, "groups": groups, "conv": 4, "norm_groups": groups}}
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff},
+           "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}
+    return {"architecture": "Felovik", "vocab": vocab, "width": width, "max_positions": max_positions, "norm": {"eps": 1e-5},
+            "embedding": {"scale": 1.0}, "postln_alpha": 1.0,
+            "layers": [{"type": "parallel", "mixer": mixer, "mlp": dense if i % dense_every == 0 else moe} for i in range(n_layers)]}
+
+
+# The third architecture: a test-sized model and the layer sizes of a 2B-class model (random weights; no
+# checkpoint of this design exists).
+CATALOG += [
+    ModelEntry("felovik-tiny", felovik_config(320, 96, 4, 2, 32, 4, 16, 16, 2, 160, 8, 48, 2, 4, max_positions=512),
+               default_ctx=512, init_norm_jitter=True),
+    ModelEntry("felovik-2b", felovik_config(32768, 2048, 16, 8, 128, 32, 64, 128, 8, 6144, 32, 1024, 4, 24)),
+]
+
 _BY_NAME = {e.name: e for e in CATALOG}
 
 

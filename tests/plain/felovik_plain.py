@@ -46,10 +46,25 @@ def query_temperature(positions: torch.Tensor, coef: float, every: int) -> torch
     return 1.0 + coef * torch.log(steps.to(torch.float64) + 1.0)
 
 
+def attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> torch.Tensor:
+    """Causal softmax attention of one sequence: ``q [T, H, d]``, ``k [T, G, d]``, ``v [T, G, dv]``; query
+    head ``a`` uses key/value head ``a // (H / G)``; position ``i`` sees every ``j <= i``."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    out = torch.zeros(T, H, v.shape[2], dtype=q.dtype)
+    visible = torch.arange(T)[None, :] <= torch.arange(T)[:, None]
+    for a in range(H):
+        g = a // (H // G)
+        s = (q[:, a] @ k[:, g].T) * scale
+        s = s.masked_fill(~visible, float("-inf"))
+        out[:, a] = torch.softmax(s, dim=-1) @ v[:, g]
+    return out
+
+
 def gated_attention(h: torch.Tensor, t: Dict[str, torch.Tensor], pre: str, m: Dict, eps: float) -> torch.Tensor:
-    """Causal softmax attention with grouped key/value heads and no rotation: queries and keys
-    are divided by their root mean square per head, the query is stretched with its position,
-    and the heads are gated by a sigmoid of a projection of ``h`` before the output matrix."""
+    """Attention without rotation: queries and keys are divided by their root mean square per head,
+    the query is stretched with its position, and the heads are gated by a sigmoid of a projection
+    of ``h`` before the output matrix."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = (h @ t[pre + "q"].T).reshape(T, H, d)
@@ -59,14 +74,7 @@ def gated_attention(h: torch.Tensor, t: Dict[str, torch.Tensor], pre: str, m: Di
     if m.get("q_temp") is not None:
         temp = query_temperature(torch.arange(T), m["q_temp"]["coef"], m["q_temp"]["every"]).to(h.dtype)
         q = q * temp[:, None, None]
-    out = torch.zeros(T, H, dv, dtype=h.dtype)
-    visible = torch.arange(T)[None, :] <= torch.arange(T)[:, None]
-    for a in range(H):
-        g = a // (H // G)
-        s = (q[:, a] @ k[:, g].T) * m["scale"]
-        s = s.masked_fill(~visible, float("-inf"))
-        p = torch.softmax(s, dim=-1)
-        out[:, a] = p @ v[:, g]
+    out = attend(q, k, v, m["scale"])
     gate = torch.sigmoid(h @ t[pre + "g"].T)
     return (out.reshape(T, H * dv) * gate) @ t[pre + "o"].T
 
@@ -82,32 +90,45 @@ def causal_conv(u: torch.Tensor, w: torch.Tensor, b: torch.Tensor) -> torch.Tens
     return out
 
 
+def recurrence(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
+               a_log: torch.Tensor, d_skip: torch.Tensor) -> torch.Tensor:
+    """``x [T, H, P]``, ``B`` and ``C [T, G, N]``, ``dt_raw [T, H]``.  Per head ``a`` (group
+    ``a // (H / G)``): ``dt = softplus(dt_raw + dt_bias)``, ``S <- exp(-exp(A_log) dt) S + dt B x^T``
+    (``S`` is ``N x P``, zero at the start), ``y = S^T C + D x``."""
+    T, Hs, P = x.shape
+    G, N = B.shape[1], B.shape[2]
+    dt = softplus(dt_raw + dt_bias)
+    decay = torch.exp(-torch.exp(a_log)[None, :] * dt)        # [T, H]
+    y = torch.zeros(T, Hs, P, dtype=x.dtype)
+    for a in range(Hs):
+        g = a // (Hs // G)
+        S = torch.zeros(N, P, dtype=x.dtype)
+        for r in range(T):
+            S = decay[r, a] * S + dt[r, a] * torch.outer(B[r, g], x[r, a])
+            y[r, a] = S.T @ C[r, g] + d_skip[a] * x[r, a]
+    return y
+
+
+def gated_part_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, parts: int, eps: float) -> torch.Tensor:
+    """``y * silu(z)`` first, then every one of the ``parts`` equal parts of a row divided by its own root
+    mean square, times ``w``."""
+    T, n = y.shape
+    v = y * silu(z)
+    return rms(v.reshape(T, parts, n // parts), eps).reshape(T, n) * w
+
+
 def state_space(h: torch.Tensor, t: Dict[str, torch.Tensor], pre: str, m: Dict, eps: float) -> torch.Tensor:
-    """The recurrence with a scalar decay per head: ``S <- exp(-exp(A_log) dt) S + dt B x^T``,
-    ``y = S^T C + D x``; inputs through a short causal convolution and silu; the output gated by
-    silu(z), normed in equal parts, and projected."""
+    """The input projection gives ``[z | x | B | C | dt]``; x, B and C pass the short causal convolution
+    and silu, then the recurrence; its output is gated by z, normed in parts and projected."""
     T = h.shape[0]
     Hs, P, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
     inner = Hs * P
     proj = h @ t[pre + "in"].T
     z, xbc, dt = proj[:, :inner], proj[:, inner:2 * inner + 2 * G * N], proj[:, 2 * inner + 2 * G * N:]
     xbc = silu(causal_conv(xbc, t[pre + "conv"], t[pre + "conv.b"]))
-    x = xbc[:, :inner].reshape(T, Hs, P)
-    B = xbc[:, inner:inner + G * N].reshape(T, G, N)
-    C = xbc[:, inner + G * N:].reshape(T, G, N)
-    dt = softplus(dt + t[pre + "dt_bias"])
-    decay = torch.exp(-torch.exp(t[pre + "A_log"])[None, :] * dt)        # [T, Hs]
-    y = torch.zeros(T, Hs, P, dtype=h.dtype)
-    for a in range(Hs):
-        g = a // (Hs // G)
-        S = torch.zeros(N, P, dtype=h.dtype)
-        for r in range(T):
-            S = decay[r, a] * S + dt[r, a] * torch.outer(B[r, g], x[r, a])
-            y[r, a] = S.T @ C[r, g] + t[pre + "D"][a] * x[r, a]
-    y = y.reshape(T, inner) * silu(z)
-    parts = m["norm_groups"]
-    y = rms(y.reshape(T, parts, inner // parts), eps).reshape(T, inner) * t[pre + "norm"]
-    return y @ t[pre + "o"].T
+    y = recurrence(xbc[:, :inner].reshape(T, Hs, P), xbc[:, inner:inner + G * N].reshape(T, G, N),
+                   xbc[:, inner + G * N:].reshape(T, G, N), dt, t[pre + "dt_bias"], t[pre + "A_log"], t[pre + "D"])
+    return gated_part_norm(y.reshape(T, inner), z, t[pre + "norm"], m["norm_groups"], eps) @ t[pre + "o"].T
 
 
 def parallel_mixer(h: torch.Tensor, t: Dict[str, torch.Tensor], pre: str, m: Dict, eps: float) -> torch.Tensor:
@@ -117,19 +138,25 @@ def parallel_mixer(h: torch.Tensor, t: Dict[str, torch.Tensor], pre: str, m: Dic
     return 0.5 * (norm(left, t[pre + "left.out"], eps) + norm(right, t[pre + "right.out"], eps))
 
 
+def limited_gate(g: torch.Tensor, u: torch.Tensor, limit: Optional[float]) -> torch.Tensor:
+    """``g <- min(g, limit)``, ``u <- clamp(u, -limit, limit)``, then ``g sigmoid(1.702 g) (u + 1)``."""
+    if limit is not None:
+        g, u = torch.clamp(g, max=limit), torch.clamp(u, min=-limit, max=limit)
+    return g * torch.sigmoid(1.702 * g) * (u + 1.0)
+
+
 def dense_ff(h: torch.Tensor, t: Dict[str, torch.Tensor], pre: str, m: Dict) -> torch.Tensor:
-    """``g = min(W_gate h, limit)``, ``u = clamp(W_up h, -limit, limit)``,
-    ``W_down (g sigmoid(1.702 g) (u + 1))``."""
-    limit = m["limit"]
-    g = torch.clamp(h @ t[pre + "gate"].T, max=limit)
-    u = torch.clamp(h @ t[pre + "up"].T, min=-limit, max=limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ t[pre + "down"].T
+    return limited_gate(h @ t[pre + "gate"].T, h @ t[pre + "up"].T, m.get("limit")) @ t[pre + "down"].T
 
 
 def route(h: torch.Tensor, w_router: torch.Tensor, r: Dict):
+    return choose(h @ w_router.T, r)
+
+
+def choose(logits: torch.Tensor, r: Dict):
     """Softmax over all experts; only experts of the ``keep`` best groups (a group's score is its
     largest) can be chosen; the ``top`` best of those, their scores divided by their sum."""
-    s = torch.softmax(h @ w_router.T, dim=-1)
+    s = torch.softmax(logits, dim=-1)
     T, E = s.shape
     allowed = torch.ones(T, E, dtype=torch.bool)
     groups = r.get("groups")
