@@ -2,7 +2,7 @@
 """Decode and prefill speed of the Qwen3 shapes with random bfloat16 weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--model qwen3-8b|qwen3-14b|qwen3-32b]
-    python bench.py --design dokulix [--design-size 2b|8b] [--layers N]
+    python bench.py --design dokulix|felovik [--design-size 2b|8b] [--layers N]
 
 The default run is the Qwen3-8B shape.  A step is one decode step of a batch of 8 sequences,
 each with a 2,048-token random prompt in the cache (context length 4,096): the engine's step
@@ -26,6 +26,9 @@ attention in turn, relu-gated feed-forward) and a Qwen3 model of the same width,
 feed-forward and number of layers, both with random weights; for each the throughput of a
 2,048-token prompt step and of decode steps of a batch of 8 over 2,048-token prompts, and per kind
 of launch its time against its analytical minimum (``efficiency``), from launch-by-launch timing.
+``--design felovik`` does the same for a Felovik model (in every layer a gated attention and a
+state-space recurrence on the same input, norms after the sums; dense feed-forwards and routed experts
+in turn, four of 32 experts a token, as many active feed-forward weights as the dense layer has).
 
 The workloads follow the reference's bench (rocml-cli/src/cmd_bench.rs:79-243): synthetic
 prompts, greedy, no stop token, warm-up first; times are taken around synchronised steps.
@@ -55,8 +58,22 @@ DESIGN_SIZES = {
 }
 
 
-def design_configs(size: dict, n_layers: int):
-    """config.json of the Dokulix model and of the Qwen3 model of equal size."""
+def felovik_config(z: dict, n_layers: int):
+    """config.json of the Felovik model of these layer sizes: recurrence heads of 64 values and a state of 128
+    with an inner width equal to the model's, 32 experts of a quarter of the dense feed-forward each."""
+    mixer = {"left": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+                      "scale": z["dim"] ** -0.5, "q_temp": {"coef": 0.1, "every": 1024}},
+             "right": {"heads": z["width"] // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}}
+    dense = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 4},
+           "router": {"experts": 32, "top": 4, "groups": {"count": 4, "keep": 2}}}
+    return {"architecture": "Felovik", "vocab": z["vocab"], "width": z["width"], "max_positions": 40960, "norm": {"eps": 1e-5},
+            "embedding": {"scale": 1.0}, "postln_alpha": 1.0,
+            "layers": [{"type": "parallel", "mixer": mixer, "mlp": dense if i % 2 == 0 else moe} for i in range(n_layers)]}
+
+
+def design_configs(size: dict, n_layers: int, design: str = "dokulix"):
+    """config.json of the design's model and of the Qwen3 model of equal size."""
     z = size
     att = {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
            "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
@@ -72,6 +89,8 @@ def design_configs(size: dict, n_layers: int):
             "num_attention_heads": z["heads"], "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
             "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False,
             "max_position_embeddings": 40960, "hidden_act": "silu", "attention_bias": False}
+    if design == "felovik":
+        return felovik_config(z, n_layers), qwen
     return dokulix, qwen
 
 
@@ -93,7 +112,7 @@ def run_design(args) -> int:
     rng = np.random.default_rng(0)
     dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     results = {}
-    for name, raw in zip((args.design, "qwen3"), design_configs(DESIGN_SIZES[args.design_size], n_layers)):
+    for name, raw in zip((args.design, "qwen3"), design_configs(DESIGN_SIZES[args.design_size], n_layers, args.design)):
         model = random_model(raw, seed=0, dtype=args.dtype, device="cuda:0")
         vocab = model.spec.vocab
         engine = Engine(model, max_tokens=batch * CONTEXT, max_seqs=batch, max_step_tokens=8192)
@@ -162,7 +181,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the further points")
     ap.add_argument("--prefill-runs", type=int, default=3)
-    ap.add_argument("--design", default=None, choices=["dokulix"],
+    ap.add_argument("--design", default=None, choices=["dokulix", "felovik"],
                     help="measure this architecture at real layer sizes beside the closest Qwen3 shape, instead of the default workload")
     ap.add_argument("--design-size", default="2b", choices=sorted(DESIGN_SIZES), help="layer sizes for --design")
     ap.add_argument("--skip-prompts", action="store_true",

@@ -124,6 +124,24 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
     "gate_heads": ("output gate", lambda x, x_stride, gate, out, n_heads, n: (2 * _nbytes(out) + out.numel() * 4, 4 * out.numel())),
     "sigmoid_gate": ("output gate", lambda y, gate: (2 * _nbytes(y) + y.numel() * 4, 4 * y.numel())),
     "splitk_reduce": ("sum of K pieces", _tensor_args_cost()),
+    "sum_norm": ("residual sum and norm", lambda x, branches, gains, gain, eps, **kw: (
+        2 * _nbytes(x) + _nbytes(*branches) + _nbytes(kw.get("copy")), 4 * x.numel() * (1 + len(branches)))),
+    "convert": ("copy in the compute type", lambda x, out: (_nbytes(x, out), 0)),
+    "causal_conv": ("causal convolution", lambda u, col0, n_channels, w, bias, state, token_seq, cu, slots, out, **kw: (
+        2 * _nbytes(out) + _nbytes(w), 2 * out.numel() * w.shape[1])),
+    "ssd_scan": ("recurrence", lambda xbc, dt_src, dt_col0, dt_bias, a_log, d_skip, state, cu, slots, y, n_heads, head_dim,
+                 n_state, n_groups: (_nbytes(xbc, y) + 2 * slots.numel() * n_heads * head_dim * n_state * 4,
+                                     4 * xbc.shape[0] * n_heads * head_dim * n_state)),
+    "gated_part_norm": ("gated norm in parts", lambda y, z, z_col0, gain, out, parts, eps: (
+        2 * _nbytes(y) + _nbytes(out), 8 * y.numel())),
+    "moe_route": ("choice of experts", lambda logits, top, groups, sum_eps, chosen, weight: (_nbytes(logits, chosen, weight),
+                                                                                            4 * logits.numel())),
+    "moe_plan": ("plan of the experts' rows", lambda chosen, n_experts, plan: (3 * _nbytes(chosen), 0)),
+    "moe_gemm": ("experts' products", lambda a, w, out, plan, top, gather, w2=None, **kw: (
+        min(w.shape[0], out.shape[0]) * w.shape[1] * w.shape[2] * w.element_size() * (2 if w2 is not None else 1)
+        + out.shape[0] * (w.shape[2] * a.element_size() + w.shape[1] * out.element_size()),
+        2 * out.shape[0] * w.shape[1] * w.shape[2] * (2 if w2 is not None else 1))),
+    "moe_combine": ("weighted sum of experts", lambda y, plan, weight, out, **kw: (_nbytes(y, out), 2 * y.numel())),
     "argmax": ("argmax", _tensor_args_cost()),
     "sample": ("sampling", lambda logits, *a, **kw: (_nbytes(logits), 0)),
 }
