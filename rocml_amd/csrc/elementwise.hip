@@ -1028,6 +1028,93 @@ sum_norm_kernel(float* __restrict__ x, SumNormBranches br, float alpha, float c,
     }
 }
 
+// The same for rows of up to 8192 values that are a multiple of 4 and at most two branches: the row and
+// the branches stay in registers and all loads are issued at once (a decode step's few rows would
+// otherwise wait for one load after the other, pass after pass).
+template <typename TC, int VEC, int NB>
+__global__ void __launch_bounds__(EW_BLOCK)
+sum_norm_vec_kernel(float* __restrict__ x, SumNormBranches br, float alpha, float c, const float* __restrict__ gain,
+                    float eps, int n, TC* __restrict__ copy) {
+    __shared__ float scratch[EW_BLOCK / WAVE];
+    size_t row = (size_t)blockIdx.x * n;
+    int nv = n / 4;
+    float4 xv[VEC], yv[NB][VEC], gv[NB][VEC], fg[VEC];
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        int i = threadIdx.x + j * EW_BLOCK;
+        bool ok = i < nv;
+        xv[j] = (ok && alpha != 0.f) ? ((const float4*)(x + row))[i] : zero4;
+        fg[j] = (ok && gain) ? ((const float4*)gain)[i] : zero4;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            yv[b][j] = ok ? ((const float4*)(br.y[b] + row))[i] : zero4;
+            gv[b][j] = (ok && br.gain[b]) ? ((const float4*)br.gain[b])[i] : zero4;
+        }
+    }
+    float inv[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        inv[b] = 1.f;
+        if (br.gain[b]) {
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+                ss = fmaf(yv[b][j].x, yv[b][j].x, ss); ss = fmaf(yv[b][j].y, yv[b][j].y, ss);
+                ss = fmaf(yv[b][j].z, yv[b][j].z, ss); ss = fmaf(yv[b][j].w, yv[b][j].w, ss);
+            }
+            inv[b] = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        float4 sum = zero4;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            float4 v = yv[b][j];
+            if (br.gain[b]) {
+                sum.x += v.x * inv[b] * gv[b][j].x; sum.y += v.y * inv[b] * gv[b][j].y;
+                sum.z += v.z * inv[b] * gv[b][j].z; sum.w += v.w * inv[b] * gv[b][j].w;
+            } else {
+                sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+            }
+        }
+        float4 sv;
+        sv.x = alpha != 0.f ? fmaf(alpha, xv[j].x, c * sum.x) : c * sum.x;
+        sv.y = alpha != 0.f ? fmaf(alpha, xv[j].y, c * sum.y) : c * sum.y;
+        sv.z = alpha != 0.f ? fmaf(alpha, xv[j].z, c * sum.z) : c * sum.z;
+        sv.w = alpha != 0.f ? fmaf(alpha, xv[j].w, c * sum.w) : c * sum.w;
+        xv[j] = sv;
+        ss = fmaf(sv.x, sv.x, ss); ss = fmaf(sv.y, sv.y, ss); ss = fmaf(sv.z, sv.z, ss); ss = fmaf(sv.w, sv.w, ss);
+    }
+    float r = gain ? 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps) : 1.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+        int i = threadIdx.x + j * EW_BLOCK;
+        if (i >= nv) continue;
+        float4 v = xv[j];
+        if (gain) { v.x *= r * fg[j].x; v.y *= r * fg[j].y; v.z *= r * fg[j].z; v.w *= r * fg[j].w; }
+        ((float4*)(x + row))[i] = v;
+        if (copy) store4(copy + row + 4 * (size_t)i, v.x, v.y, v.z, v.w);
+    }
+}
+
+template <typename TC>
+static bool launch_sum_norm_vec(float* x, const SumNormBranches& br, float alpha, float c, const float* gain, float eps, int n,
+                                TC* copy, int n_rows, hipStream_t stream) {
+    int vec = ceil_div(n / 4, EW_BLOCK);
+#define SNV(V_, NB_) sum_norm_vec_kernel<TC, V_, NB_><<<n_rows, EW_BLOCK, 0, stream>>>(x, br, alpha, c, gain, eps, n, copy)
+#define SNV_BY_NB(V_) { if (br.n == 1) SNV(V_, 1); else SNV(V_, 2); }
+    if (vec <= 1) SNV_BY_NB(1)
+    else if (vec <= 2) SNV_BY_NB(2)
+    else if (vec <= 4) SNV_BY_NB(4)
+    else SNV_BY_NB(8)
+#undef SNV_BY_NB
+#undef SNV
+    return true;
+}
+
 ROCML_EXPORT int rocml_sum_norm(float* x, int n_rows, int n, float alpha, float c, int n_branches,
                                 const float* const* ys, const float* const* gains, const float* gain, float eps,
                                 void* copy, int copy_dtype, hipStream_t stream) {
@@ -1041,6 +1128,13 @@ ROCML_EXPORT int rocml_sum_norm(float* x, int n_rows, int n, float alpha, float 
         ROCML_REQUIRE(ys[b], "sum_norm: branch %d has no values", b);
         br.y[b] = ys[b];
         br.gain[b] = gains[b];
+    }
+    ROCML_REQUIRE(!copy || copy_dtype == ROCML_F32 || copy_dtype == ROCML_BF16, "sum_norm: unknown dtype code %d", copy_dtype);
+    if (n % 4 == 0 && n <= 4 * EW_BLOCK * RN_MAX_VEC && n_branches <= 2) {
+        if (!copy || copy_dtype == ROCML_F32) launch_sum_norm_vec<float>(x, br, alpha, c, gain, eps, n, (float*)copy, n_rows, stream);
+        else launch_sum_norm_vec<bf16_t>(x, br, alpha, c, gain, eps, n, (bf16_t*)copy, n_rows, stream);
+        ROCML_CHECK_LAUNCH("sum_norm");
+        return 0;
     }
     if (!copy || copy_dtype == ROCML_F32)
         sum_norm_kernel<float><<<n_rows, EW_BLOCK, 0, stream>>>(x, br, alpha, c, gain, eps, n, (float*)copy);

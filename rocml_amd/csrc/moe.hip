@@ -11,7 +11,7 @@
 
 ROCML_LAST_ERROR_FN(moe)
 
-constexpr int MOE_TM = 64;            // rows of a tile of the experts' products
+constexpr int MOE_TM = 128;           // rows of a tile of the experts' products
 constexpr int RT_MAX_PER_LANE = 8;    // experts per lane of the routing wave: at most 512 experts
 constexpr int RT_BLOCK = 256;
 
@@ -226,28 +226,31 @@ struct MoeGemmArgs {
 __device__ __forceinline__ float moe_silu(float z) { return z / (1.0f + expf(-z)); }
 
 // Any sizes and types, fused multiply-add in 32-bit: the whole 32-bit path and shapes the
-// matrix-core kernel refuses.  64 x 64 outputs per block, 4 x 4 per thread, K staged 16 at a time.
+// matrix-core kernel refuses.  64 x 64 outputs at a time (a tile's rows in MOE_TM / 64 passes), 4 x 4
+// per thread, K staged 16 at a time.
 template <typename TA, typename TW, typename TO, bool DUAL>
 __global__ void __launch_bounds__(256)
 moe_gemm_plain_kernel(MoeGemmArgs g) {
     int tile = blockIdx.y;
     if (tile >= g.n_tiles[0]) return;
-    __shared__ float as[16][MOE_TM + 4];
+    __shared__ float as[16][64 + 4];
     __shared__ float ws[16][64 + 4];
     __shared__ float ws2[DUAL ? 16 : 1][64 + 4];
-    __shared__ int src[MOE_TM];
-    int expert = g.tiles[2 * tile], r0 = g.tiles[2 * tile + 1];
+    __shared__ int src[64];
+    int expert = g.tiles[2 * tile], tile_r0 = g.tiles[2 * tile + 1];
     int r_end = g.offsets[expert + 1];
     int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
     int n0 = blockIdx.x * 64;
-    if (tid < MOE_TM) {
+    const TA* a = (const TA*)g.a;
+    const TW* w = (const TW*)g.w + (size_t)expert * g.w_expert_stride;
+    const TW* w2 = DUAL ? (const TW*)g.w2 + (size_t)expert * g.w_expert_stride : nullptr;
+  for (int r0 = tile_r0; r0 < min(tile_r0 + MOE_TM, r_end); r0 += 64) {
+    __syncthreads();
+    if (tid < 64) {
         int r = r0 + tid;
         src[tid] = r < r_end ? (g.order ? g.order[r] / g.top : r) : -1;
     }
     __syncthreads();
-    const TA* a = (const TA*)g.a;
-    const TW* w = (const TW*)g.w + (size_t)expert * g.w_expert_stride;
-    const TW* w2 = DUAL ? (const TW*)g.w2 + (size_t)expert * g.w_expert_stride : nullptr;
     float acc[4][4] = {}, acc2[DUAL ? 4 : 1][4] = {};
     for (int k0 = 0; k0 < g.k; k0 += 16) {
 #pragma unroll
@@ -294,10 +297,12 @@ moe_gemm_plain_kernel(MoeGemmArgs g) {
             Elem<TO>::store((TO*)g.out + (size_t)r * g.ldo + gn, v);
         }
     }
+  }
 }
 
 // bfloat16 operands on the matrix cores (v_mfma_f32_16x16x32_bf16), 32-bit sums.  Four waves a
-// block; a wave owns 16 of the block's 64 columns and all 64 rows.  The rows' activations (gathered)
+// block; a wave owns 16 of the block's 64 columns and all MOE_TM rows (a weight fragment from memory
+// meets MOE_TM / 16 row fragments from LDS).  The rows' activations (gathered)
 // go through LDS 64 values of K at a time; a wave's weight fragments come straight from memory
 // (a lane reads 16 bytes of one weight row), requested a stage ahead.  K must be a multiple of 8.
 typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8_t;
@@ -328,23 +333,26 @@ moe_gemm_mfma_kernel(MoeGemmArgs g) {
     const bf16_t* w = (const bf16_t*)g.w + wrow;
     const bf16_t* w2 = DUAL ? (const bf16_t*)g.w2 + wrow : nullptr;
     int kq = (lane >> 4) * 8;              // the lane's 8 K values inside a 32-wide step
-    // the two 16-byte pieces of the activations this thread stages: rows tid / 8 and tid / 8 + 32
+    // the 16-byte pieces of the activations this thread stages: rows tid / 8 + 32 i
+    constexpr int MT = MOE_TM / 16, XP = MOE_TM / 32;
     int piece_k = (tid & 7) * 8;
-    int row_a = src[tid >> 3], row_b = src[(tid >> 3) + 32];
-    moe_f32x4_t acc[4], acc2[DUAL ? 4 : 1];
+    int rows_x[XP];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[i] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < XP; ++i) rows_x[i] = src[(tid >> 3) + 32 * i];
+    moe_f32x4_t acc[MT], acc2[DUAL ? MT : 1];
 #pragma unroll
-    for (int i = 0; i < (DUAL ? 4 : 1); ++i) acc2[i] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < MT; ++i) acc[i] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < (DUAL ? MT : 1); ++i) acc2[i] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
     const moe_u32x4_t zero = {0u, 0u, 0u, 0u};
     int n_stages = (g.k + MG_KC - 1) / MG_KC;
-    moe_u32x4_t xa, xb, wf[2], wf2[DUAL ? 2 : 1];
+    moe_u32x4_t xr[XP], wf[2], wf2[DUAL ? 2 : 1];
 #define MG_LOAD(stage_)                                                                                        \
     {                                                                                                          \
         int kb_ = (stage_) * MG_KC;                                                                            \
         int gk_ = kb_ + piece_k;                                                                               \
-        xa = (row_a >= 0 && gk_ < g.k) ? *(const moe_u32x4_t*)(a + (size_t)row_a * g.lda + gk_) : zero;        \
-        xb = (row_b >= 0 && gk_ < g.k) ? *(const moe_u32x4_t*)(a + (size_t)row_b * g.lda + gk_) : zero;        \
+        _Pragma("unroll") for (int i = 0; i < XP; ++i)                                                         \
+            xr[i] = (rows_x[i] >= 0 && gk_ < g.k) ? *(const moe_u32x4_t*)(a + (size_t)rows_x[i] * g.lda + gk_) : zero; \
         _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                        \
             int wk_ = min(kb_ + j * 32 + kq, g.k - 8);       /* beyond K the activations are zero */           \
             wf[j] = *(const moe_u32x4_t*)(w + wk_);                                                            \
@@ -354,8 +362,8 @@ moe_gemm_mfma_kernel(MoeGemmArgs g) {
     MG_LOAD(0)
     for (int s = 0; s < n_stages; ++s) {
         int buf = s & 1;
-        xs[buf][(tid >> 3) * MG_ROW + (tid & 7)] = xa;
-        xs[buf][((tid >> 3) + 32) * MG_ROW + (tid & 7)] = xb;
+#pragma unroll
+        for (int i = 0; i < XP; ++i) xs[buf][((tid >> 3) + 32 * i) * MG_ROW + (tid & 7)] = xr[i];
         moe_u32x4_t wc[2], wc2[DUAL ? 2 : 1];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -368,7 +376,7 @@ moe_gemm_mfma_kernel(MoeGemmArgs g) {
         for (int j = 0; j < 2; ++j) {
             moe_bf16x8_t wa = __builtin_bit_cast(moe_bf16x8_t, wc[j]);
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt) {
+            for (int mt = 0; mt < MT; ++mt) {
                 moe_bf16x8_t xv = __builtin_bit_cast(moe_bf16x8_t, xs[buf][(mt * 16 + (lane & 15)) * MG_ROW + j * 4 + (lane >> 4)]);
                 acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xv, acc[mt], 0, 0, 0);
                 if (DUAL)
@@ -380,7 +388,7 @@ moe_gemm_mfma_kernel(MoeGemmArgs g) {
 #undef MG_LOAD
     // acc[mt][e]: row mt * 16 + (lane & 15) of the tile, column n0 + (lane >> 4) * 4 + e
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
         int r = r0 + mt * 16 + (lane & 15);
         if (r >= r_end) continue;
 #pragma unroll

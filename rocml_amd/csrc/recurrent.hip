@@ -44,6 +44,43 @@ causal_conv_kernel(const float* __restrict__ u, int ldu, int col0, int n_channel
     out[idx] = silu ? rc_silu(acc) : acc;
 }
 
+// Four neighbouring channels per thread, as 16-byte pieces (channels, first column and row strides are
+// multiples of 4): a quarter of the loads and of the index arithmetic.
+typedef float cv_f4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(RC_BLOCK)
+causal_conv_vec_kernel(const float* __restrict__ u, int ldu, int col0, int n_channels, int taps,
+                       const float* __restrict__ w, const float* __restrict__ bias, const float* __restrict__ state,
+                       const int* __restrict__ token_seq, const int* __restrict__ cu_seqlens,
+                       const int* __restrict__ seq_slots, float* __restrict__ out, long long total4, int silu) {
+    long long idx = (long long)blockIdx.x * RC_BLOCK + threadIdx.x;
+    if (idx >= total4) return;
+    int c4 = n_channels / 4;
+    int t = (int)(idx / c4), c = (int)(idx - (long long)t * c4) * 4;
+    int b = token_seq[t];
+    int local = t - cu_seqlens[b];
+    const float* st = state + (size_t)seq_slots[b] * (taps - 1) * n_channels;
+    cv_f4 acc = bias ? *(const cv_f4*)(bias + c) : cv_f4{0.f, 0.f, 0.f, 0.f};
+    cv_f4 v[CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        if (j >= taps) break;
+        int src = local - (taps - 1) + j;
+        v[j] = src >= 0 ? *(const cv_f4*)(u + (size_t)(t - (taps - 1) + j) * ldu + col0 + c)
+                        : *(const cv_f4*)(st + (size_t)(taps - 1 + src) * n_channels + c);
+    }
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        if (j >= taps) break;
+        acc.x = fmaf(w[(size_t)c * taps + j], v[j].x, acc.x);
+        acc.y = fmaf(w[(size_t)(c + 1) * taps + j], v[j].y, acc.y);
+        acc.z = fmaf(w[(size_t)(c + 2) * taps + j], v[j].z, acc.z);
+        acc.w = fmaf(w[(size_t)(c + 3) * taps + j], v[j].w, acc.w);
+    }
+    if (silu) { acc.x = rc_silu(acc.x); acc.y = rc_silu(acc.y); acc.z = rc_silu(acc.z); acc.w = rc_silu(acc.w); }
+    *(cv_f4*)(out + (size_t)t * n_channels + c) = acc;
+}
+
 // The state after the step: the last taps - 1 inputs of each sequence, taken from the step's
 // tokens and, where the step brought fewer, from the old state.  Runs after the outputs.
 __global__ void __launch_bounds__(RC_BLOCK)
@@ -81,8 +118,13 @@ ROCML_EXPORT int rocml_causal_conv(const float* u, int ldu, int col0, int n_toke
     ROCML_REQUIRE(u && w && out && token_seq && cu_seqlens && seq_slots && (taps == 1 || state), "causal_conv: missing arguments");
     if (n_tokens == 0 || n_seqs == 0) return 0;
     long long total = (long long)n_tokens * n_channels;
-    causal_conv_kernel<<<ceil_div(total, RC_BLOCK), RC_BLOCK, 0, stream>>>(u, ldu, col0, n_channels, taps, w, bias, state, token_seq,
-                                                                           cu_seqlens, seq_slots, out, total, silu);
+    bool vec = n_channels % 4 == 0 && col0 % 4 == 0 && ldu % 4 == 0 && (((uintptr_t)u | (uintptr_t)out | (uintptr_t)state | (uintptr_t)bias) & 15) == 0;
+    if (vec)
+        causal_conv_vec_kernel<<<ceil_div(total / 4, RC_BLOCK), RC_BLOCK, 0, stream>>>(u, ldu, col0, n_channels, taps, w, bias, state,
+                                                                                       token_seq, cu_seqlens, seq_slots, out, total / 4, silu);
+    else
+        causal_conv_kernel<<<ceil_div(total, RC_BLOCK), RC_BLOCK, 0, stream>>>(u, ldu, col0, n_channels, taps, w, bias, state, token_seq,
+                                                                               cu_seqlens, seq_slots, out, total, silu);
     ROCML_CHECK_LAUNCH("causal_conv");
     if (taps > 1) {
         long long st_total = (long long)n_seqs * n_channels;
@@ -99,76 +141,178 @@ ROCML_EXPORT int rocml_causal_conv(const float* u, int ldu, int col0, int n_toke
 //     dt = softplus(raw + dt_bias[a]),  S <- exp(-exp(A_log[a]) dt) S + dt B_t x_t^T,
 //     y_t = S^T C_t + D[a] x_t.
 // The columns of S (one per value p) do not depend on each other: a block takes one sequence, one
-// head and SC_PT values and walks the sequence's tokens in order; thread (p, r) keeps the state
-// entries n = r, r + SC_R, ... of column p in registers and the SC_R threads of a column add up
-// their parts of S^T C by butterfly.  Tokens come through LDS tc at a time (at most SC_MAX_TC).  State layout:
-// [slot, H, P, N].
-constexpr int SC_R = 16, SC_PT = RC_BLOCK / SC_R, SC_MAX_TC = 32;
+// head and SC_PT values and walks the sequence's tokens in order.  Thread (pair of columns, r) keeps
+// the state entries n = r * NI .. r * NI + NI - 1 of its two columns in registers (2 NI numbers); the
+// 16 threads of a column pair sit in one row of 16 lanes and add up their parts of S^T C with four
+// cross-lane additions inside the row, in a fixed order.  Tokens come through LDS tc at a time, B and
+// C rows padded with zeros to 16 NI numbers so that a thread reads its NI numbers as whole vectors.
+// State layout: [slot, H, P, N].
+typedef float sc_f4 __attribute__((ext_vector_type(4)));      // 16 bytes as a native vector
+constexpr int SC_R = 16, SC_PP = 2, SC_PT = RC_BLOCK / SC_R * SC_PP, SC_MAX_TC = 32, SC_U = 4;
 
-template <int NI>
+// sum over the 16 lanes of a row, the same in every lane: lanes 1 apart, 2 apart, mirrored inside a
+// half row, mirrored inside the row
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));
+    return v;
+}
+
+template <int NI, bool VEC>
 __global__ void __launch_bounds__(RC_BLOCK)
 ssd_scan_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict__ dtsrc, int lddt, int dt_col0,
                 const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
                 float* __restrict__ state, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slots,
                 float* __restrict__ y, int n_heads, int head_dim, int n_state, int n_groups, int tc) {
-    extern __shared__ float sc_smem[];
-    float* bs = sc_smem;                       // [tc][N]
-    float* cs = bs + tc * n_state;             // [tc][N]
-    float* xs = cs + tc * n_state;             // [tc][SC_PT]
+    extern __shared__ float4 sc_smem4[];
+    constexpr int NP = SC_R * NI;              // padded length of a B or C row
+    float* bs = (float*)sc_smem4;              // [tc][NP]
+    float* cs = bs + tc * NP;                  // [tc][NP]
+    float* xs = cs + tc * NP;                  // [tc][SC_PT]
     float* ys = xs + tc * SC_PT;               // [tc][SC_PT]
-    float* dts = ys + tc * SC_PT;              // [tc]
-    float* decs = dts + tc;                    // [tc]
+    float* dts = ys + tc * SC_PT;              // [tc][2]: step size, decay
     int p0 = blockIdx.x * SC_PT, head = blockIdx.y, b = blockIdx.z;
     int tid = threadIdx.x, r = tid % SC_R, pl = tid / SC_R;
-    int p = p0 + pl;
-    bool p_ok = p < head_dim;
     int group = head / (n_heads / n_groups);
     int inner = n_heads * head_dim;
     int first = cu_seqlens[b], n_tok = cu_seqlens[b + 1] - first;
-    float* st = state + (((size_t)seq_slots[b] * n_heads + head) * head_dim + (p_ok ? p : 0)) * n_state;
-    float s[NI];
+    float* st_head = state + ((size_t)seq_slots[b] * n_heads + head) * head_dim * n_state;
+    float s[SC_PP][NI];
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-        int n = r + i * SC_R;
-        s[i] = (p_ok && n < n_state) ? st[n] : 0.f;
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            int n = r * NI + i;
+            s[j][i] = (p < head_dim && n < n_state) ? st_head[(size_t)p * n_state + n] : 0.f;
+        }
     }
     float a_rate = expf(a_log[head]), bias = dt_bias[head], skip = d_skip[head];
+    // VEC (rows of the inputs and the sizes are multiples of 4 numbers): a chunk's operands are asked
+    // for as 16-byte pieces, all at once, while the chunk before it is worked on, and reach LDS when
+    // that is done; a block is alone on its CU for most launches, and a chunk's loads one after the
+    // other, with nothing to do meanwhile, would take longer than its arithmetic.
+    constexpr int PF = VEC ? (SC_MAX_TC * NP / 4 + RC_BLOCK - 1) / RC_BLOCK : 1;
+    sc_f4 pre_b[PF], pre_c[PF], pre_x;
+    float pre_dt = 0.f;
+    const sc_f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    pre_x = zero4;
+#define SC_PREFETCH(c0_)                                                                                         \
+    {                                                                                                            \
+        int nt_ = min(tc, n_tok - (c0_));                                                                        \
+        _Pragma("unroll") for (int j = 0; j < PF; ++j) {                                                         \
+            int i4 = tid + j * RC_BLOCK, tt = i4 / (NP / 4), n = (i4 - tt * (NP / 4)) * 4;                       \
+            bool ok = tt < nt_ && n < n_state;                                                                   \
+            const float* row = xbc + (size_t)(first + (c0_) + (ok ? tt : 0)) * ldx + inner + (size_t)group * n_state + (ok ? n : 0); \
+            pre_b[j] = ok ? *(const sc_f4*)row : zero4;                                                         \
+            pre_c[j] = ok ? *(const sc_f4*)(row + (size_t)n_groups * n_state) : zero4;                          \
+        }                                                                                                        \
+        {                                                                                                        \
+            int tt = tid / (SC_PT / 4), pp = (tid - tt * (SC_PT / 4)) * 4;                                       \
+            bool ok = tt < nt_ && p0 + pp < head_dim;                                                            \
+            pre_x = ok ? *(const sc_f4*)(xbc + (size_t)(first + (c0_) + tt) * ldx + (size_t)head * head_dim + p0 + pp) : zero4; \
+        }                                                                                                        \
+        pre_dt = tid < nt_ ? dtsrc[(size_t)(first + (c0_) + tid) * lddt + dt_col0 + head] : 0.f;                 \
+    }
+    if (VEC && n_tok > 0) SC_PREFETCH(0)
     for (int c0 = 0; c0 < n_tok; c0 += tc) {
         int nt = min(tc, n_tok - c0);
+        int nt_up = (nt + SC_U - 1) / SC_U * SC_U;
         __syncthreads();                          // the previous chunk's outputs have been written out
-        for (int i = tid; i < nt * n_state; i += RC_BLOCK) {
-            int tt = i / n_state, n = i - tt * n_state;
-            const float* row = xbc + (size_t)(first + c0 + tt) * ldx + inner + (size_t)group * n_state + n;
-            bs[i] = row[0];
-            cs[i] = row[(size_t)n_groups * n_state];
-        }
-        for (int i = tid; i < nt * SC_PT; i += RC_BLOCK) {
-            int tt = i / SC_PT, pp = i - tt * SC_PT;
-            xs[i] = p0 + pp < head_dim ? xbc[(size_t)(first + c0 + tt) * ldx + (size_t)head * head_dim + p0 + pp] : 0.f;
-        }
-        if (tid < nt) {
-            float dt = rc_softplus(dtsrc[(size_t)(first + c0 + tid) * lddt + dt_col0 + head] + bias);
-            dts[tid] = dt;
-            decs[tid] = expf(-a_rate * dt);
-        }
-        __syncthreads();
-        for (int tt = 0; tt < nt; ++tt) {
-            float dec = decs[tt], xv = xs[tt * SC_PT + pl];
-            float dtx = dts[tt] * xv;
-            const float* bt = bs + tt * n_state;
-            const float* ct = cs + tt * n_state;
-            float part = 0.f;
+        if (VEC) {
+            // (rows past the chunk's end were fetched as zeros: a step of zero and a decay of one leave the state alone)
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                int n = r + i * SC_R;
-                if (n < n_state) {
-                    s[i] = fmaf(dec, s[i], dtx * bt[n]);
-                    part = fmaf(s[i], ct[n], part);
+            for (int j = 0; j < PF; ++j) {
+                int i4 = tid + j * RC_BLOCK;
+                if (i4 < tc * (NP / 4)) {
+                    ((sc_f4*)bs)[i4] = pre_b[j];
+                    ((sc_f4*)cs)[i4] = pre_c[j];
                 }
             }
+            if (tid < tc * (SC_PT / 4)) ((sc_f4*)xs)[tid] = pre_x;
+            if (tid < tc) {
+                float dt = tid < nt ? rc_softplus(pre_dt + bias) : 0.f;
+                dts[2 * tid] = dt;
+                dts[2 * tid + 1] = tid < nt ? expf(-a_rate * dt) : 1.f;
+            }
+            __syncthreads();
+            if (c0 + tc < n_tok) SC_PREFETCH(c0 + tc)
+        } else {
+            for (int i = tid; i < nt * NP; i += RC_BLOCK) {
+                int tt = i / NP, n = i - tt * NP;
+                const float* row = xbc + (size_t)(first + c0 + tt) * ldx + inner + (size_t)group * n_state + n;
+                bool ok = n < n_state;
+                bs[i] = ok ? row[0] : 0.f;
+                cs[i] = ok ? row[(size_t)n_groups * n_state] : 0.f;
+            }
+            for (int i = tid; i < nt * SC_PT; i += RC_BLOCK) {
+                int tt = i / SC_PT, pp = i - tt * SC_PT;
+                xs[i] = p0 + pp < head_dim ? xbc[(size_t)(first + c0 + tt) * ldx + (size_t)head * head_dim + p0 + pp] : 0.f;
+            }
+            if (tid < nt) {
+                float dt = rc_softplus(dtsrc[(size_t)(first + c0 + tid) * lddt + dt_col0 + head] + bias);
+                dts[2 * tid] = dt;
+                dts[2 * tid + 1] = expf(-a_rate * dt);
+            }
+            // tokens that fill the chunk up to a multiple of SC_U: a step of zero and a decay of one
+            for (int i = nt * NP + tid; i < nt_up * NP; i += RC_BLOCK) { bs[i] = 0.f; cs[i] = 0.f; }
+            for (int i = nt * SC_PT + tid; i < nt_up * SC_PT; i += RC_BLOCK) xs[i] = 0.f;
+            if (tid >= nt && tid < nt_up) { dts[2 * tid] = 0.f; dts[2 * tid + 1] = 1.f; }
+            __syncthreads();
+        }
+        // SC_U tokens at a time: all their operands are read before the first is used and their sums
+        // across lanes run side by side, so that a wave alone on its SIMD does not wait for every
+        // load and every cross-lane step in turn.  Tokens past the chunk's end leave the state as it is.
+        for (int t0 = 0; t0 < nt; t0 += SC_U) {
+            float2 dd[SC_U], xv[SC_U];
+            float bv[SC_U][NI], cv[SC_U][NI];
 #pragma unroll
-            for (int off = SC_R / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
-            if (r == 0) ys[tt * SC_PT + pl] = fmaf(skip, xv, part);
+            for (int u = 0; u < SC_U; ++u) {
+                int tt = t0 + u;
+                dd[u] = *(const float2*)(dts + 2 * tt);
+                xv[u] = *(const float2*)(xs + tt * SC_PT + pl * SC_PP);
+                const float* bt = bs + tt * NP + r * NI;
+                const float* ct = cs + tt * NP + r * NI;
+                if (NI % 4 == 0) {
+#pragma unroll
+                    for (int i = 0; i < NI; i += 4) {
+                        float4 b4 = *(const float4*)(bt + i), c4 = *(const float4*)(ct + i);
+                        bv[u][i] = b4.x; bv[u][i + 1] = b4.y; bv[u][i + 2] = b4.z; bv[u][i + 3] = b4.w;
+                        cv[u][i] = c4.x; cv[u][i + 1] = c4.y; cv[u][i + 2] = c4.z; cv[u][i + 3] = c4.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NI; ++i) { bv[u][i] = bt[i]; cv[u][i] = ct[i]; }
+                }
+            }
+            float part0[SC_U], part1[SC_U];
+#pragma unroll
+            for (int u = 0; u < SC_U; ++u) {
+                float dec = dd[u].y, dtx0 = dd[u].x * xv[u].x, dtx1 = dd[u].x * xv[u].y;
+                float q0 = 0.f, q1 = 0.f;
+#pragma unroll
+                for (int i = 0; i < NI; ++i) {
+                    s[0][i] = fmaf(dec, s[0][i], dtx0 * bv[u][i]);
+                    s[1][i] = fmaf(dec, s[1][i], dtx1 * bv[u][i]);
+                    q0 = fmaf(s[0][i], cv[u][i], q0);
+                    q1 = fmaf(s[1][i], cv[u][i], q1);
+                }
+                part0[u] = q0;
+                part1[u] = q1;
+            }
+#pragma unroll
+            for (int u = 0; u < SC_U; ++u) {
+                part0[u] = row16_sum(part0[u]);
+                part1[u] = row16_sum(part1[u]);
+            }
+            if (r == 0) {
+#pragma unroll
+                for (int u = 0; u < SC_U; ++u)
+                    *(float2*)(ys + (t0 + u) * SC_PT + pl * SC_PP) =
+                        make_float2(fmaf(skip, xv[u].x, part0[u]), fmaf(skip, xv[u].y, part1[u]));
+            }
         }
         __syncthreads();
         for (int i = tid; i < nt * SC_PT; i += RC_BLOCK) {
@@ -176,11 +320,14 @@ ssd_scan_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict_
             if (p0 + pp < head_dim) y[(size_t)(first + c0 + tt) * inner + (size_t)head * head_dim + p0 + pp] = ys[i];
         }
     }
-    if (p_ok) {
+#undef SC_PREFETCH
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            int n = r + i * SC_R;
-            if (n < n_state) st[n] = s[i];
+            int n = r * NI + i;
+            if (p < head_dim && n < n_state) st_head[(size_t)p * n_state + n] = s[j][i];
         }
     }
 }
@@ -199,21 +346,33 @@ ROCML_EXPORT int rocml_ssd_scan(const float* xbc, int ldx, const float* dtsrc, i
     ROCML_REQUIRE(n_seqs >= 0 && n_seqs < 65536 && n_heads < 65536, "ssd_scan: too many sequences or heads for one launch");
     if (n_seqs == 0 || n_tokens == 0) return 0;
     dim3 grid(ceil_div(head_dim, SC_PT), n_heads, n_seqs);
-    int tc = n_state <= 128 ? SC_MAX_TC : SC_MAX_TC / 2;          // 64 KB of LDS at most
-    size_t lds = (size_t)(2 * tc * n_state + 2 * tc * SC_PT + 2 * tc) * sizeof(float);
     int ni = ceil_div(n_state, SC_R);
+    ni = ni <= 4 ? ni : ni <= 6 ? 6 : ni <= 8 ? 8 : ni <= 12 ? 12 : 16;
+    int tc = ni <= 8 ? SC_MAX_TC : SC_MAX_TC / 2;          // 48 KB of LDS at most
+    size_t lds = (size_t)(2 * tc * SC_R * ni + 2 * tc * SC_PT + 2 * tc) * sizeof(float);
+    // whole 16-byte pieces: every row of x, B and C starts on a multiple of 4 numbers and ends on one
+    bool vec = ldx % 4 == 0 && head_dim % 4 == 0 && n_state % 4 == 0 && ((uintptr_t)xbc & 15) == 0;
 #define SCAN(NI_)                                                                                              \
-    ssd_scan_kernel<NI_><<<grid, RC_BLOCK, lds, stream>>>(xbc, ldx, dtsrc, lddt, dt_col0, dt_bias, a_log, d_skip, \
-                                                          state, cu_seqlens, seq_slots, y, n_heads, head_dim,  \
-                                                          n_state, n_groups, tc)
-    if (ni <= 1) SCAN(1);
-    else if (ni <= 2) SCAN(2);
-    else if (ni <= 3) SCAN(3);
-    else if (ni <= 4) SCAN(4);
-    else if (ni <= 6) SCAN(6);
-    else if (ni <= 8) SCAN(8);
-    else if (ni <= 12) SCAN(12);
-    else SCAN(16);
+    {                                                                                                          \
+        if (vec)                                                                                               \
+            ssd_scan_kernel<NI_, true><<<grid, RC_BLOCK, lds, stream>>>(xbc, ldx, dtsrc, lddt, dt_col0, dt_bias, a_log, d_skip, \
+                                                                        state, cu_seqlens, seq_slots, y, n_heads, head_dim, \
+                                                                        n_state, n_groups, tc);                \
+        else                                                                                                   \
+            ssd_scan_kernel<NI_, false><<<grid, RC_BLOCK, lds, stream>>>(xbc, ldx, dtsrc, lddt, dt_col0, dt_bias, a_log, d_skip, \
+                                                                         state, cu_seqlens, seq_slots, y, n_heads, head_dim, \
+                                                                         n_state, n_groups, tc);               \
+    }
+    switch (ni) {
+        case 1: SCAN(1); break;
+        case 2: SCAN(2); break;
+        case 3: SCAN(3); break;
+        case 4: SCAN(4); break;
+        case 6: SCAN(6); break;
+        case 8: SCAN(8); break;
+        case 12: SCAN(12); break;
+        default: SCAN(16); break;
+    }
 #undef SCAN
     ROCML_CHECK_LAUNCH("ssd_scan");
     return 0;

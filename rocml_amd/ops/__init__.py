@@ -996,7 +996,7 @@ def gated_part_norm(y: torch.Tensor, z: torch.Tensor, z_col0: int, gain: torch.T
 
 
 # ---- experts -----------------------------------------------------------------------------
-MOE_TILE_ROWS = 64
+MOE_TILE_ROWS = 128
 
 
 def moe_max_tiles(n_pairs: int, n_experts: int) -> int:

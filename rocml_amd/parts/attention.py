@@ -169,20 +169,34 @@ class Attention(Mixer):
             return 0
         return ops.decode_splits(step.n_tokens * self.spec.n_kv_heads, self.n_cus, min(cache.block_table.shape[1], 64))
 
-    def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
+    def input_weight(self) -> Optional[torch.Tensor]:
+        # only the path of the norm-and-rotation kernel, which takes rows of any stride; and the
+        # projection must start at the buffer's first column
+        return self.w_qkv if self.separate_q and not self.spec.bias else None
+
+    def adopt_input_weight(self, view: torch.Tensor) -> None:
+        self.w_qkv = view
+
+    def forward(self, step, xn, x_accum, cache, owns_cache: bool, projected=None) -> None:
         s = self.spec
         n = step.n_tokens
         ws = step.workspace
         rows = self.q_dim + self.kv_dim + self.v_dim + self.g_dim if owns_cache else self.q_dim
         if s.gate and not owns_cache:
             raise ConfigError("a gated attention layer that reads another layer's cache is not supported")
-        qkv = ws.get("attn.qkv", (n, rows), torch.float32)
         scratch = ws.scratch()
-        # (the decode kernel that reads the projection adds four partial sums in one trip to memory
-        # and further ones one after the other: K is cut into few pieces for it)
-        # (the gate's columns are read where they lie: the product is then completed)
-        splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=not s.gate,
-                          max_splits=ops.FUSED_DECODE_SPLITS if self._fused_decode(step) else 0)
+        if projected is not None:
+            qkv, first = projected
+            if first != 0 or not owns_cache or qkv.shape[1] < rows:
+                raise ConfigError("the attention takes a projection that starts at the buffer's first column")
+            splits = 0
+        else:
+            qkv = ws.get("attn.qkv", (n, rows), torch.float32)
+            # (the decode kernel that reads the projection adds four partial sums in one trip to memory
+            # and further ones one after the other: K is cut into few pieces for it)
+            # (the gate's columns are read where they lie: the product is then completed)
+            splits = ops.gemm(xn, self.w_qkv[:rows], qkv, workspace=scratch, defer=not s.gate,
+                              max_splits=ops.FUSED_DECODE_SPLITS if self._fused_decode(step) else 0)
         if splits:      # the product's split-K partial sums; the next kernel adds them
             qkv = scratch[:splits * n * rows * 4].view(torch.float32).view(splits, n, rows)
         cos = sin = None
@@ -230,7 +244,7 @@ class Attention(Mixer):
                               max_len=step.max_len, n_splits=self._decode_splits(step, cache),
                               v_head_dim=self.v_head_dim, chunk=s.chunk, slopes=self.slopes, sink=s.sink)
         if s.gate:
-            ops.sigmoid_gate(o, qkv[:, rows - self.g_dim:])
+            ops.sigmoid_gate(o, qkv[:, rows - self.g_dim:rows])
         if self.b_o is not None:
             ws.flush_pending()
             ops.add_row_vector(x_accum, self.b_o)

@@ -177,6 +177,14 @@ class Mixer(Part):
     def cache_request(self) -> Optional[Any]:
         return None
 
+    def input_weight(self) -> Optional[torch.Tensor]:
+        """The matrix ``[rows, hidden]`` of the mixer's first product, if ``forward`` can be handed that
+        product's result (``projected=(buffer, first column)``: 32-bit ``[tokens, width]``, the mixer's
+        columns starting at ``first column``) instead of forming it.  A mixer that runs beside others on
+        the same input then shares one product with them.  None: the mixer multiplies itself.
+        ``adopt_input_weight(view)`` replaces the matrix by an equal one that lives inside a larger."""
+        return None
+
     def forward(self, step: Any, xn: torch.Tensor, x_accum: torch.Tensor, cache: Any,
                 owns_cache: bool) -> None:
         """Adds the mixer's output for the step's tokens into ``x_accum`` (32-bit,

@@ -2,7 +2,9 @@
 every branch's output normed over the model width with a gain of its own.
 
 A branch is any registered mixer, built from its spec; each keeps what it needs in the cache
-through a part of a composite request.  The branches' outputs stay in buffers of their own: a block
+through a part of a composite request.  Branches whose first step is a product with the input
+(``input_weight``) share one product over their matrices laid one under the other, and each finds
+its columns in the result.  The branches' outputs stay in buffers of their own: a block
 that norms after its sum takes them as they are (``branches``) and does the branches' norms, their
 sum, the residual sum and its own norm in one kernel; in any other block ``forward`` adds the
 weighted sum to the stream.
@@ -37,6 +39,8 @@ class ParallelMixer(Mixer):
         self.prompt_graph_safe = all(getattr(c, "prompt_graph_safe", False) for c in self.children.values())
         self.kernel_families = tuple(f for c in self.children.values() for f in getattr(c, "kernel_families", ()))
         self.gains: Dict[str, torch.Tensor] = {}
+        self.w_in = None              # the branches' first matrices as one, if they share a product
+        self.first_column: Dict[str, int] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         specs = {}
@@ -52,6 +56,18 @@ class ParallelMixer(Mixer):
             own = {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
             self.gains[name] = own.pop("out_norm.weight")
             child.bind(own)
+        # One product for all branches that can take its result: their matrices one under the other, each
+        # branch's own matrix replaced by its rows of the whole (no second copy stays).
+        takers = [(name, child) for name, child in self.children.items()
+                  if getattr(child, "input_weight", None) is not None and child.input_weight() is not None]
+        if len(takers) >= 2 and len({w.dtype for w in (c.input_weight() for _, c in takers)}) == 1:
+            self.w_in = torch.cat([child.input_weight() for _, child in takers], dim=0).contiguous()
+            at = 0
+            for name, child in takers:
+                n_rows = child.input_weight().shape[0]
+                self.first_column[name] = at
+                child.adopt_input_weight(self.w_in[at:at + n_rows])
+                at += n_rows
 
     def cache_request(self) -> CompositeRequest:
         return CompositeRequest(tuple(child.cache_request() for child in self.children.values()))
@@ -70,10 +86,17 @@ class ParallelMixer(Mixer):
         before = rs.overwrite
         views = cache.parts if cache is not None else (None,) * len(self.children)
         outs: List[torch.Tensor] = []
+        proj = None
+        if self.w_in is not None and owns_cache:
+            proj = ws.get("parallel.proj", (step.n_tokens, self.w_in.shape[0]), torch.float32)
+            ops.gemm(xn, self.w_in, proj, workspace=ws.scratch())
         for i, (name, child) in enumerate(self.children.items()):
             y = ws.get(f"parallel.y{i}", (step.n_tokens, self.spec.hidden), torch.float32)
             rs.overwrite = True
-            child.forward(step, xn, y, views[i], owns_cache)
+            if proj is not None and name in self.first_column:
+                child.forward(step, xn, y, views[i], owns_cache, projected=(proj, self.first_column[name]))
+            else:
+                child.forward(step, xn, y, views[i], owns_cache)
             ws.flush_pending()
             outs.append(y)
         rs.overwrite = before

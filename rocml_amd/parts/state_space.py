@@ -77,23 +77,32 @@ class StateSpaceMixer(Mixer):
         size = 2 if self.dtype == torch.bfloat16 else 4
         return n_tokens * ((self.proj_dim + self.conv_channels + self.inner) * 4 + self.inner * size)
 
-    def forward(self, step, xn, x_accum, cache, owns_cache: bool) -> None:
+    def input_weight(self) -> Optional[torch.Tensor]:
+        return self.w_in
+
+    def adopt_input_weight(self, view: torch.Tensor) -> None:
+        self.w_in = view
+
+    def forward(self, step, xn, x_accum, cache, owns_cache: bool, projected=None) -> None:
         if not owns_cache:
             raise ConfigError("a recurrent layer cannot run on another layer's state")
         s = self.spec
         n = step.n_tokens
         ws = step.workspace
         state, conv_state = cache.parts
-        proj = ws.get("ssm.proj", (n, self.proj_dim), torch.float32)
-        ops.gemm(xn, self.w_in, proj, workspace=ws.scratch())
+        if projected is not None:        # the projection is columns c0 .. of a product shared with other mixers
+            proj, c0 = projected
+        else:
+            proj, c0 = ws.get("ssm.proj", (n, self.proj_dim), torch.float32), 0
+            ops.gemm(xn, self.w_in, proj, workspace=ws.scratch())
         xbc = ws.get("ssm.xbc", (n, self.conv_channels), torch.float32)
-        ops.causal_conv(proj, self.inner, self.conv_channels, self.conv_w, self.conv_b, conv_state.state, step.token_seq,
+        ops.causal_conv(proj, c0 + self.inner, self.conv_channels, self.conv_w, self.conv_b, conv_state.state, step.token_seq,
                         step.cu_seqlens, step.seq_slots, xbc, silu=True)
         y = ws.get("ssm.y", (n, self.inner), torch.float32)
-        ops.ssd_scan(xbc, proj, 2 * self.inner + 2 * self.bc, self.dt_bias, self.a_log, self.d_skip, state.state,
+        ops.ssd_scan(xbc, proj, c0 + 2 * self.inner + 2 * self.bc, self.dt_bias, self.a_log, self.d_skip, state.state,
                      step.cu_seqlens, step.seq_slots, y, s.n_heads, s.head_dim, s.state, s.groups)
         gated = ws.get("ssm.gated", (n, self.inner), self.dtype)
-        ops.gated_part_norm(y, proj, 0, self.norm_gain, gated, s.norm_groups, s.eps)
+        ops.gated_part_norm(y, proj, c0, self.norm_gain, gated, s.norm_groups, s.eps)
         stream(step).add_product(gated, self.w_out, x_accum)
 
 

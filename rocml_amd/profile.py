@@ -129,9 +129,9 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
     "convert": ("copy in the compute type", lambda x, out: (_nbytes(x, out), 0)),
     "causal_conv": ("causal convolution", lambda u, col0, n_channels, w, bias, state, token_seq, cu, slots, out, **kw: (
         2 * _nbytes(out) + _nbytes(w), 2 * out.numel() * w.shape[1])),
-    "ssd_scan": ("recurrence", lambda xbc, dt_src, dt_col0, dt_bias, a_log, d_skip, state, cu, slots, y, n_heads, head_dim,
+    "ssd_scan": ("recurrence (32-bit vector work)", lambda xbc, dt_src, dt_col0, dt_bias, a_log, d_skip, state, cu, slots, y, n_heads, head_dim,
                  n_state, n_groups: (_nbytes(xbc, y) + 2 * slots.numel() * n_heads * head_dim * n_state * 4,
-                                     4 * xbc.shape[0] * n_heads * head_dim * n_state)),
+                                     4 * xbc.shape[0] * n_heads * head_dim * n_state, PEAK_FLOPS[torch.float32])),
     "gated_part_norm": ("gated norm in parts", lambda y, z, z_col0, gain, out, parts, eps: (
         2 * _nbytes(y) + _nbytes(out), 8 * y.numel())),
     "moe_route": ("choice of experts", lambda logits, top, groups, sum_eps, chosen, weight: (_nbytes(logits, chosen, weight),
@@ -236,7 +236,9 @@ class OpProfiler:
             start.record()
             result = fn(*a, **kw)
             end.record()
-            b, f = cost(*a, **kw)
+            b, f, *peak = cost(*a, **kw)
+            if peak:        # work that cannot run at the profiler's peak rate (32-bit vector arithmetic under a
+                f = f * self.peak_flops / peak[0]      # bfloat16 model): its operations count as so many at that peak
             name = label(*a, **kw) if callable(label) else label       # (a label may depend on the call)
             self._records.append((self.phase, name, int(b), int(f), start, end))
             return result

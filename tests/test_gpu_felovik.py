@@ -26,7 +26,9 @@ TOL = {"float32": 1e-4}
 # pin most of them against the plain implementation and all of them against each other (a fault of the
 # cache, the state or the batch shows between two bfloat16 runs that should agree).
 BF16_MOST = {"A": (0.9, 6e-2), "B": (0.9, 6e-2), "C": (0.5, 1e-1)}
-BF16_SAME = (0.98, 3e-2)
+# (A and C run the same kernels whatever the step's shape and agree to the last bit; B's head sizes take the
+# matrix-core attention, whose prompt and single-token kernels round differently)
+BF16_SAME = {"A": (0.98, 3e-2), "B": (0.9, 6e-2), "C": (0.98, 3e-2)}
 LENGTHS = {"A": [1, 2, 21, 66, 150, 211], "B": [3, 64, 65, 131, 262], "C": [1, 8, 30, 77]}
 
 
@@ -68,9 +70,9 @@ def _fits(got, ref, dtype, name) -> bool:
     return float(torch.quantile(_errors(got, ref), q)) < tol
 
 
-def _same(got, other, most=BF16_SAME) -> bool:
+def _same(got, other, name) -> bool:
     """Whether two bfloat16 runs of the same tokens agree."""
-    q, tol = most
+    q, tol = BF16_SAME[name]
     return float(torch.quantile(_errors(got, other), q)) < tol
 
 
@@ -88,7 +90,7 @@ def test_whole_tail_and_batches(models, name, dtype):
         # the last 100 tokens one by one: state, convolution memory and keys all come from the cache
         tail = helpers.run_tail_by_one(engine, p, 100)
         assert _fits(tail, refs[i], dtype, name), f"tail, length {len(p)}"
-        assert dtype == "float32" or _same(tail, whole[i]), f"tail against whole, length {len(p)}"
+        assert dtype == "float32" or _same(tail, whole[i], name), f"tail against whole, length {len(p)}"
     # batches of unequal requests, twice, so that slots, pages and states are used again; the second time in another order
     for order in (list(range(len(prompts))), list(reversed(range(len(prompts))))):
         batch = [prompts[i] for i in order]
@@ -96,7 +98,7 @@ def test_whole_tail_and_batches(models, name, dtype):
         got = helpers.run_batch(engine, batch, n_prefill)
         for j, i in enumerate(order):
             assert _fits(got[j], refs[i], dtype, name), f"batch, request of length {len(prompts[i])}"
-            assert dtype == "float32" or _same(got[j], whole[i]), f"batch against alone, length {len(prompts[i])}"
+            assert dtype == "float32" or _same(got[j], whole[i], name), f"batch against alone, length {len(prompts[i])}"
     engine.cache.check()
     assert not engine.cache.lengths
 
@@ -126,7 +128,7 @@ def test_prompts_cut_into_portions(models, piece, dtype):
     for p, ref in zip(prompts, refs):
         got = helpers.run_whole(engine, p)
         assert _fits(got, ref, dtype, "A"), f"pieces of {piece}, length {len(p)}"
-        assert dtype == "float32" or _same(got, helpers.run_whole(uncut, p)), f"pieces of {piece} against the whole, length {len(p)}"
+        assert dtype == "float32" or _same(got, helpers.run_whole(uncut, p), "A"), f"pieces of {piece} against the whole, length {len(p)}"
     # three unequal requests in one step that is cut across them
     got = helpers.run_batch(engine, prompts, [len(p) for p in prompts])
     for g, ref in zip(got, refs):
@@ -176,8 +178,8 @@ def test_long_portions_on_top_of_a_cache_with_unequal_starts(models, dtype):
     if dtype == "bfloat16":
         # (portions of other sizes take other product kernels, whose sums round differently, and 760 sharp
         # positions amplify that: most positions, not nearly all)
-        assert _same(torch.cat(out_a), helpers.run_whole(engine, a), BF16_MOST["B"])
-        assert _same(torch.cat(out_b), helpers.run_whole(engine, b), BF16_MOST["B"])
+        assert _same(torch.cat(out_a), helpers.run_whole(engine, a), "B")
+        assert _same(torch.cat(out_b), helpers.run_whole(engine, b), "B")
     engine.cache.check()
 
 
@@ -292,5 +294,5 @@ def test_prompt_steps_of_one_shape_are_replayed(models):
         ref = _ref(cfg, tensors, p)
         got = helpers.run_tail_by_one(engine, p, 3)
         assert _fits(got, ref, "bfloat16", "B"), f"prompt {k}"
-        assert _same(got, helpers.run_whole(_engine(path, "bfloat16", use_graphs=False), p)), f"prompt {k} against a run without graphs"
+        assert _same(got, helpers.run_whole(_engine(path, "bfloat16", use_graphs=False), p), "B"), f"prompt {k} against a run without graphs"
     assert any(key[0] == "prompt" and entry[1] is not None for key, entry in engine._graphs.items()), "a prompt shape was recorded"

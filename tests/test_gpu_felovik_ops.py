@@ -136,15 +136,17 @@ def _pieces(total, sizes):
     return out
 
 
+@pytest.mark.parametrize("C,lead", [(37, 11), (40, 12)])
 @pytest.mark.parametrize("taps", [1, 2, 4, 8])
-def test_convolution_carried_through_pieces(taps):
+def test_convolution_carried_through_pieces(taps, C, lead):
     """Two sequences in slots 5 and 2 of 7, fed in pieces of unequal sizes (some shorter than the taps);
     then slot 5 again from zero for a third sequence."""
     from rocml_amd import ops
-    C, lead = 37, 11
+    # (37 channels behind 11 others in rows of 51: one channel a thread; 40 behind 12 in rows of 56: four)
+    tail = 3 if C % 4 else 4
     g = _gen(taps)
     w, b = torch.randn(C, taps, generator=g), torch.randn(C, generator=g)
-    seqs = [torch.randn(n, lead + C + 3, generator=g) for n in (50, 23)]
+    seqs = [torch.randn(n, lead + C + tail, generator=g) for n in (50, 23)]
     state = torch.zeros((7, taps - 1, C), dtype=torch.float32, device=DEV)
     state[1].fill_(9.0)                 # another sequence's memory must not leak in
     slots = [5, 2]
@@ -170,7 +172,7 @@ def test_convolution_carried_through_pieces(taps):
     assert taps == 1 or float(state[1].min()) == 9.0
     # the slot is handed out again: the cache zeroes it, and a new sequence starts from nothing
     state[5].zero_()
-    third = torch.randn(6, lead + C + 3, generator=g)
+    third = torch.randn(6, lead + C + tail, generator=g)
     out = torch.empty((6, C), dtype=torch.float32, device=DEV)
     ops.causal_conv(third.to(DEV), lead, C, w.to(DEV), b.to(DEV), state, torch.zeros(6, dtype=torch.int32, device=DEV),
                     torch.tensor([0, 6], dtype=torch.int32, device=DEV), torch.tensor([5], dtype=torch.int32, device=DEV), out)
@@ -334,10 +336,11 @@ def test_experts_products_and_weighted_sum(T, w, ff, E, top, dtype, tol):
         _close(hid, hid2.double().cpu(), 2e-2)
 
 
-def test_sum_and_norm():
+@pytest.mark.parametrize("n", [72, 70, 2048, 9000])
+def test_sum_and_norm(n):
     from rocml_amd import ops
     g = _gen(12)
-    n, T, eps = 72, 9, 1e-4
+    T, eps = 9, 1e-4
     x, a, b = torch.randn(T, n, generator=g), torch.randn(T, n, generator=g) * 5, torch.randn(T, n, generator=g) * 0.1
     wa, wb, w = torch.randn(n, generator=g), torch.randn(n, generator=g), torch.randn(n, generator=g)
     # two branches, each normed with its gain, half their sum, the scaled stream, the norm after it
