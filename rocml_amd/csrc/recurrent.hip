@@ -18,8 +18,8 @@ __device__ __forceinline__ float rc_silu(float z) { return z / (1.0f + expf(-z))
 __device__ __forceinline__ float rc_softplus(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
 // ---- causal convolution per channel ------------------------------------------------
-// out[t, c] = act(bias[c] + sum_j w[c, j] * in(t - (taps - 1) + j, c)): the last column of w is
-// the current token's.  Inputs before the step's first token of a sequence come from the
+// out[t, c] = act(bias[c] + sum_j w[j, c] * in(t - (taps - 1) + j, c)): w is [taps, C] (a tap's weights of
+// neighbouring channels lie side by side, as the threads that read them do), its last row the current token's.  Inputs before the step's first token of a sequence come from the
 // sequence's state [slot, taps - 1, C] (its last taps - 1 inputs, oldest first; zeros at the
 // start).  u is [T, ldu] 32-bit and the channels are its columns col0 .. col0 + C - 1.
 constexpr int CONV_MAX_TAPS = 8;
@@ -39,7 +39,7 @@ causal_conv_kernel(const float* __restrict__ u, int ldu, int col0, int n_channel
     for (int j = 0; j < taps; ++j) {
         int src = local - (taps - 1) + j;
         float v = src >= 0 ? u[(size_t)(t - (taps - 1) + j) * ldu + col0 + c] : st[(size_t)(taps - 1 + src) * n_channels + c];
-        acc = fmaf(w[(size_t)c * taps + j], v, acc);
+        acc = fmaf(w[(size_t)j * n_channels + c], v, acc);
     }
     out[idx] = silu ? rc_silu(acc) : acc;
 }
@@ -72,10 +72,11 @@ causal_conv_vec_kernel(const float* __restrict__ u, int ldu, int col0, int n_cha
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j) {
         if (j >= taps) break;
-        acc.x = fmaf(w[(size_t)c * taps + j], v[j].x, acc.x);
-        acc.y = fmaf(w[(size_t)(c + 1) * taps + j], v[j].y, acc.y);
-        acc.z = fmaf(w[(size_t)(c + 2) * taps + j], v[j].z, acc.z);
-        acc.w = fmaf(w[(size_t)(c + 3) * taps + j], v[j].w, acc.w);
+        cv_f4 wj = *(const cv_f4*)(w + (size_t)j * n_channels + c);
+        acc.x = fmaf(wj.x, v[j].x, acc.x);
+        acc.y = fmaf(wj.y, v[j].y, acc.y);
+        acc.z = fmaf(wj.z, v[j].z, acc.z);
+        acc.w = fmaf(wj.w, v[j].w, acc.w);
     }
     if (silu) { acc.x = rc_silu(acc.x); acc.y = rc_silu(acc.y); acc.z = rc_silu(acc.z); acc.w = rc_silu(acc.w); }
     *(cv_f4*)(out + (size_t)t * n_channels + c) = acc;
@@ -106,6 +107,44 @@ causal_conv_state_kernel(const float* __restrict__ u, int ldu, int col0, int n_c
     }
 }
 
+// A step of one token per sequence: output and new state in one launch.  A thread takes W channels
+// (1, or 4 as a 16-byte piece) of one sequence, reads its kept inputs, forms the output and moves
+// the kept inputs up by one.
+template <int W>
+__global__ void __launch_bounds__(RC_BLOCK)
+causal_conv_step_kernel(const float* __restrict__ u, int ldu, int col0, int n_channels, int taps,
+                        const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ state,
+                        const int* __restrict__ seq_slots, float* __restrict__ out, long long total, int silu) {
+    typedef float vec_t __attribute__((ext_vector_type(W)));
+    long long idx = (long long)blockIdx.x * RC_BLOCK + threadIdx.x;
+    if (idx >= total) return;
+    int cw = n_channels / W;
+    int b = (int)(idx / cw), c = (int)(idx - (long long)b * cw) * W;
+    float* st = state + (size_t)seq_slots[b] * (taps - 1) * n_channels;
+    vec_t v[CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        if (j >= taps) break;
+        v[j] = j < taps - 1 ? *(const vec_t*)(st + (size_t)j * n_channels + c) : *(const vec_t*)(u + (size_t)b * ldu + col0 + c);
+    }
+#pragma unroll
+    for (int e = 0; e < W; ++e) {
+        float acc = bias ? bias[c + e] : 0.f;
+#pragma unroll
+        for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+            if (j >= taps) break;
+            float in = W == 1 ? ((const float*)&v[j])[0] : ((const float*)&v[j])[e];
+            acc = fmaf(w[(size_t)j * n_channels + c + e], in, acc);
+        }
+        out[(size_t)b * n_channels + c + e] = silu ? rc_silu(acc) : acc;
+    }
+#pragma unroll
+    for (int j = 0; j < CONV_MAX_TAPS; ++j) {
+        if (j >= taps - 1) break;
+        *(vec_t*)(st + (size_t)j * n_channels + c) = v[j + 1];
+    }
+}
+
 ROCML_EXPORT int rocml_causal_conv(const float* u, int ldu, int col0, int n_tokens, int n_channels, int taps,
                                    const float* w, const float* bias, float* state, int n_slots,
                                    const int* token_seq, const int* cu_seqlens, const int* seq_slots, int n_seqs,
@@ -118,7 +157,19 @@ ROCML_EXPORT int rocml_causal_conv(const float* u, int ldu, int col0, int n_toke
     ROCML_REQUIRE(u && w && out && token_seq && cu_seqlens && seq_slots && (taps == 1 || state), "causal_conv: missing arguments");
     if (n_tokens == 0 || n_seqs == 0) return 0;
     long long total = (long long)n_tokens * n_channels;
-    bool vec = n_channels % 4 == 0 && col0 % 4 == 0 && ldu % 4 == 0 && (((uintptr_t)u | (uintptr_t)out | (uintptr_t)state | (uintptr_t)bias) & 15) == 0;
+    if (n_tokens == n_seqs) {
+        // one token per sequence (every sequence brings at least one): token b is sequence b's
+        bool vec4 = n_channels % 4 == 0 && col0 % 4 == 0 && ldu % 4 == 0 && (((uintptr_t)u | (uintptr_t)state) & 15) == 0;
+        if (vec4)
+            causal_conv_step_kernel<4><<<ceil_div(total / 4, RC_BLOCK), RC_BLOCK, 0, stream>>>(u, ldu, col0, n_channels, taps, w, bias,
+                                                                                             state, seq_slots, out, total / 4, silu);
+        else
+            causal_conv_step_kernel<1><<<ceil_div(total, RC_BLOCK), RC_BLOCK, 0, stream>>>(u, ldu, col0, n_channels, taps, w, bias,
+                                                                                         state, seq_slots, out, total, silu);
+        ROCML_CHECK_LAUNCH("causal_conv step");
+        return 0;
+    }
+    bool vec = n_channels % 4 == 0 && col0 % 4 == 0 && ldu % 4 == 0 && (((uintptr_t)u | (uintptr_t)out | (uintptr_t)state | (uintptr_t)bias | (uintptr_t)w) & 15) == 0;
     if (vec)
         causal_conv_vec_kernel<<<ceil_div(total / 4, RC_BLOCK), RC_BLOCK, 0, stream>>>(u, ldu, col0, n_channels, taps, w, bias, state,
                                                                                        token_seq, cu_seqlens, seq_slots, out, total / 4, silu);
@@ -415,6 +466,51 @@ gated_part_norm_kernel(const float* __restrict__ y, const float* __restrict__ z,
     }
 }
 
+// Parts of up to 2048 values that are multiples of 4: a wave takes a part (the waves of a token's block take
+// its parts in turn), keeps it in registers as 16-byte pieces and sums without a barrier.
+constexpr int GP_MAX_VEC = 8;
+
+template <typename TO, int VEC>
+__global__ void __launch_bounds__(RC_BLOCK)
+gated_part_norm_vec_kernel(const float* __restrict__ y, const float* __restrict__ z, int ldz, int z_col0,
+                           const float* __restrict__ gain, TO* __restrict__ out, int n, int parts, float eps) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    int t = blockIdx.x, wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
+    int width = n / parts, w4 = width / 4;
+    for (int part = blockIdx.y * (RC_BLOCK / WAVE) + wave; part < parts; part += gridDim.y * (RC_BLOCK / WAVE)) {
+        int i0 = part * width;
+        const float* yr = y + (size_t)t * n + i0;
+        const float* zr = z + (size_t)t * ldz + z_col0 + i0;
+        f4 v[VEC], g[VEC];
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            int i = lane + j * WAVE;
+            bool ok = i < w4;
+            f4 yy = ok ? ((const f4*)yr)[i] : f4{0.f, 0.f, 0.f, 0.f};
+            f4 zz = ok ? ((const f4*)zr)[i] : f4{0.f, 0.f, 0.f, 0.f};
+            g[j] = ok ? ((const f4*)(gain + i0))[i] : f4{0.f, 0.f, 0.f, 0.f};
+            v[j].x = yy.x * rc_silu(zz.x); v[j].y = yy.y * rc_silu(zz.y);
+            v[j].z = yy.z * rc_silu(zz.z); v[j].w = yy.w * rc_silu(zz.w);
+            ss = fmaf(v[j].x, v[j].x, ss); ss = fmaf(v[j].y, v[j].y, ss);
+            ss = fmaf(v[j].z, v[j].z, ss); ss = fmaf(v[j].w, v[j].w, ss);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        float inv = 1.0f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            int i = lane + j * WAVE;
+            if (i >= w4) continue;
+            TO* o = out + (size_t)t * n + i0 + 4 * i;
+            Elem<TO>::store(o, v[j].x * inv * g[j].x);
+            Elem<TO>::store(o + 1, v[j].y * inv * g[j].y);
+            Elem<TO>::store(o + 2, v[j].z * inv * g[j].z);
+            Elem<TO>::store(o + 3, v[j].w * inv * g[j].w);
+        }
+    }
+}
+
 ROCML_EXPORT int rocml_gated_part_norm(const float* y, const float* z, int ldz, int z_col0, const float* gain, void* out,
                                        int out_dtype, int n_rows, int n, int parts, float eps, hipStream_t stream) {
     ROCML_REQUIRE(n_rows >= 0 && n > 0 && parts > 0 && n % parts == 0, "gated_part_norm: %d values do not fall into %d equal parts", n,
@@ -422,6 +518,21 @@ ROCML_EXPORT int rocml_gated_part_norm(const float* y, const float* z, int ldz, 
     ROCML_REQUIRE(z_col0 >= 0 && ldz >= z_col0 + n, "gated_part_norm: gate rows of %d are too short", ldz);
     ROCML_REQUIRE(parts < 65536, "gated_part_norm: too many parts");
     if (n_rows == 0) return 0;
+    ROCML_REQUIRE(out_dtype == ROCML_F32 || out_dtype == ROCML_BF16, "gated_part_norm: unknown dtype code %d", out_dtype);
+    int width = n / parts;
+    if (width % 4 == 0 && width <= 4 * WAVE * GP_MAX_VEC && ldz % 4 == 0 && z_col0 % 4 == 0 &&
+        (((uintptr_t)y | (uintptr_t)z | (uintptr_t)gain) & 15) == 0) {
+        int vec = ceil_div(width / 4, WAVE);
+        dim3 vgrid(n_rows, min(ceil_div(parts, RC_BLOCK / WAVE), 1024));
+#define GPV(TO_, V_) gated_part_norm_vec_kernel<TO_, V_><<<vgrid, RC_BLOCK, 0, stream>>>(y, z, ldz, z_col0, gain, (TO_*)out, n, parts, eps)
+#define GPV_BY_VEC(TO_) { if (vec <= 1) GPV(TO_, 1); else if (vec <= 2) GPV(TO_, 2); else if (vec <= 4) GPV(TO_, 4); else GPV(TO_, 8); }
+        if (out_dtype == ROCML_F32) GPV_BY_VEC(float)
+        else GPV_BY_VEC(bf16_t)
+#undef GPV_BY_VEC
+#undef GPV
+        ROCML_CHECK_LAUNCH("gated_part_norm");
+        return 0;
+    }
     dim3 grid(n_rows, parts);
     if (out_dtype == ROCML_F32)
         gated_part_norm_kernel<float><<<grid, RC_BLOCK, 0, stream>>>(y, z, ldz, z_col0, gain, (float*)out, n, parts, eps);

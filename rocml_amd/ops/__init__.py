@@ -936,16 +936,17 @@ def causal_conv(u: torch.Tensor, col0: int, n_channels: int, w: torch.Tensor, bi
                 state: torch.Tensor, token_seq: torch.Tensor, cu_seqlens: torch.Tensor, seq_slots: torch.Tensor,
                 out: torch.Tensor, silu: bool = True) -> None:
     """Causal convolution per channel over columns ``col0 .. col0 + n_channels - 1`` of the 32-bit
-    ``u [T, ld]``: ``out[t, c] = act(bias[c] + sum_j w[c, j] in(t - (taps - 1) + j, c))``.  ``state``
+    ``u [T, ld]``: ``out[t, c] = act(bias[c] + sum_j w[j, c] in(t - (taps - 1) + j, c))``; ``w`` is
+    ``[taps, channels]``, its last row the current token's.  ``state``
     ``[slots, taps - 1, channels]`` holds every sequence's last ``taps - 1`` inputs (zeros at its
     start), is read for the inputs before the step's first token and brought up to date."""
     _dev(u, w, bias, state, token_seq, cu_seqlens, seq_slots, out)
     for t, what in ((u, "convolution input"), (w, "convolution weights"), (state, "convolution state"), (out, "convolution output")):
         _want(t, torch.float32, what)
     n_tokens, ld = u.shape
-    taps = w.shape[1]
+    taps = w.shape[0]
     n_seqs = seq_slots.numel()
-    if w.shape != (n_channels, taps) or (bias is not None and (bias.dtype != torch.float32 or bias.numel() != n_channels)):
+    if w.shape != (taps, n_channels) or (bias is not None and (bias.dtype != torch.float32 or bias.numel() != n_channels)):
         raise KernelError(f"convolution weights {tuple(w.shape)} or bias do not fit {n_channels} channels")
     if out.shape != (n_tokens, n_channels) or token_seq.numel() != n_tokens or cu_seqlens.numel() != n_seqs + 1:
         raise KernelError("convolution output or token tables do not fit the step")

@@ -59,7 +59,8 @@ class StateSpaceMixer(Mixer):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.w_in, self.w_out = tensors["in_proj.weight"], tensors["out_proj.weight"]
-        self.conv_w, self.conv_b = tensors["conv.weight"].contiguous(), tensors["conv.bias"]
+        # stored [channels, taps]; the kernels read a tap's weights of neighbouring channels side by side
+        self.conv_w, self.conv_b = tensors["conv.weight"].t().contiguous(), tensors["conv.bias"]
         self.dt_bias, self.a_log, self.d_skip = tensors["dt_bias"], tensors["A_log"], tensors["D"]
         self.norm_gain = tensors["norm.weight"]
 

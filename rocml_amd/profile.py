@@ -128,7 +128,7 @@ _COSTS: Dict[str, Tuple[str, Callable]] = {
         2 * _nbytes(x) + _nbytes(*branches) + _nbytes(kw.get("copy")), 4 * x.numel() * (1 + len(branches)))),
     "convert": ("copy in the compute type", lambda x, out: (_nbytes(x, out), 0)),
     "causal_conv": ("causal convolution", lambda u, col0, n_channels, w, bias, state, token_seq, cu, slots, out, **kw: (
-        2 * _nbytes(out) + _nbytes(w), 2 * out.numel() * w.shape[1])),
+        2 * _nbytes(out) + _nbytes(w), 2 * out.numel() * w.shape[0])),
     "ssd_scan": ("recurrence (32-bit vector work)", lambda xbc, dt_src, dt_col0, dt_bias, a_log, d_skip, state, cu, slots, y, n_heads, head_dim,
                  n_state, n_groups: (_nbytes(xbc, y) + 2 * slots.numel() * n_heads * head_dim * n_state * 4,
                                      4 * xbc.shape[0] * n_heads * head_dim * n_state, PEAK_FLOPS[torch.float32])),

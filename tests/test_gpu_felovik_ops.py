@@ -160,7 +160,7 @@ def test_convolution_carried_through_pieces(taps, C, lead):
         cu = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device=DEV)
         seq = torch.repeat_interleave(torch.arange(len(live), dtype=torch.int32), torch.tensor(counts)).to(DEV)
         out = torch.empty((sum(counts), C), dtype=torch.float32, device=DEV)
-        ops.causal_conv(u, lead, C, w.to(DEV), b.to(DEV), state, seq, cu, torch.tensor([slots[i] for i in live], dtype=torch.int32, device=DEV),
+        ops.causal_conv(u, lead, C, w.t().contiguous().to(DEV), b.to(DEV), state, seq, cu, torch.tensor([slots[i] for i in live], dtype=torch.int32, device=DEV),
                         out, silu=True)
         at = 0
         for i, n in zip(live, counts):
@@ -174,7 +174,7 @@ def test_convolution_carried_through_pieces(taps, C, lead):
     state[5].zero_()
     third = torch.randn(6, lead + C + tail, generator=g)
     out = torch.empty((6, C), dtype=torch.float32, device=DEV)
-    ops.causal_conv(third.to(DEV), lead, C, w.to(DEV), b.to(DEV), state, torch.zeros(6, dtype=torch.int32, device=DEV),
+    ops.causal_conv(third.to(DEV), lead, C, w.t().contiguous().to(DEV), b.to(DEV), state, torch.zeros(6, dtype=torch.int32, device=DEV),
                     torch.tensor([0, 6], dtype=torch.int32, device=DEV), torch.tensor([5], dtype=torch.int32, device=DEV), out)
     _close(out, plain.silu(plain.causal_conv(third[:, lead:lead + C].double(), w.double(), b.double())), 1e-5)
 
@@ -245,16 +245,17 @@ def test_far_token_through_a_slow_decay():
     _close(y, want, 2e-5)
 
 
-@pytest.mark.parametrize("n,parts", [(48, 2), (36, 36), (1024, 1), (600, 3)])
+@pytest.mark.parametrize("n,parts", [(48, 2), (36, 36), (1024, 1), (600, 3), (4096, 8), (4096, 1), (90, 5)])
 def test_gated_norm_in_parts(n, parts):
     from rocml_amd import ops
     g = _gen(n)
-    y, z, w = torch.randn(5, n, generator=g), torch.randn(5, 7 + n, generator=g) * 2, torch.randn(n, generator=g)
+    lead = 7 if n % 8 else 8            # (a gate that starts on a multiple of 4 numbers takes the vector kernel)
+    y, z, w = torch.randn(5, n, generator=g), torch.randn(5, lead + n + (0 if n % 8 else 4), generator=g) * 2, torch.randn(n, generator=g)
     y[:, :n // parts] *= 30         # one part far larger than the others: a norm over the whole row would show
-    want = plain.gated_part_norm(y.double(), z[:, 7:].double(), w.double(), parts, 1e-4)
+    want = plain.gated_part_norm(y.double(), z[:, lead:lead + n].double(), w.double(), parts, 1e-4)
     for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 1e-2)):
         out = torch.empty((5, n), dtype=dtype, device=DEV)
-        ops.gated_part_norm(y.to(DEV), z.to(DEV), 7, w.to(DEV), out, parts, 1e-4)
+        ops.gated_part_norm(y.to(DEV), z.to(DEV), lead, w.to(DEV), out, parts, 1e-4)
         _close(out, want, tol)
 
 
