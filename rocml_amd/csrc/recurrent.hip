@@ -211,6 +211,40 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
+// A thread's NI state entries of one column, n = r * NI ..: as 16-byte pieces where NI is a multiple of 4 and
+// the state is exactly 16 NI long (one load instruction of a wave then touches 16 memory lines, not 64).
+template <int NI>
+__device__ __forceinline__ void sc_load_state(float (&s)[NI], const float* col, int r, int n_state, bool p_ok) {
+    if (NI % 4 == 0 && n_state == SC_R * NI) {
+#pragma unroll
+        for (int i = 0; i < NI; i += 4) {
+            sc_f4 v = p_ok ? *(const sc_f4*)(col + r * NI + i) : sc_f4{0.f, 0.f, 0.f, 0.f};
+            s[i] = v.x; s[i + 1] = v.y; s[i + 2] = v.z; s[i + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            int n = r * NI + i;
+            s[i] = (p_ok && n < n_state) ? col[n] : 0.f;
+        }
+    }
+}
+
+template <int NI>
+__device__ __forceinline__ void sc_store_state(const float (&s)[NI], float* col, int r, int n_state, bool p_ok) {
+    if (!p_ok) return;
+    if (NI % 4 == 0 && n_state == SC_R * NI) {
+#pragma unroll
+        for (int i = 0; i < NI; i += 4) *(sc_f4*)(col + r * NI + i) = sc_f4{s[i], s[i + 1], s[i + 2], s[i + 3]};
+    } else {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            int n = r * NI + i;
+            if (n < n_state) col[n] = s[i];
+        }
+    }
+}
+
 template <int NI, bool VEC>
 __global__ void __launch_bounds__(RC_BLOCK)
 ssd_scan_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict__ dtsrc, int lddt, int dt_col0,
@@ -234,11 +268,7 @@ ssd_scan_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict_
 #pragma unroll
     for (int j = 0; j < SC_PP; ++j) {
         int p = p0 + pl * SC_PP + j;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            int n = r * NI + i;
-            s[j][i] = (p < head_dim && n < n_state) ? st_head[(size_t)p * n_state + n] : 0.f;
-        }
+        sc_load_state<NI>(s[j], st_head + (size_t)min(p, head_dim - 1) * n_state, r, n_state, p < head_dim);
     }
     float a_rate = expf(a_log[head]), bias = dt_bias[head], skip = d_skip[head];
     // VEC (rows of the inputs and the sizes are multiples of 4 numbers): a chunk's operands are asked
@@ -375,11 +405,70 @@ ssd_scan_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict_
 #pragma unroll
     for (int j = 0; j < SC_PP; ++j) {
         int p = p0 + pl * SC_PP + j;
+        sc_store_state<NI>(s[j], st_head + (size_t)min(p, head_dim - 1) * n_state, r, n_state, p < head_dim);
+    }
+}
+
+// A step of one token per sequence: the same arithmetic for that token without the chunks: a thread
+// reads its NI numbers of B and C and its two values of x straight from memory, next to its state
+// entries, and nothing waits at a barrier.  Token b is sequence b's.
+template <int NI>
+__global__ void __launch_bounds__(RC_BLOCK)
+ssd_step_kernel(const float* __restrict__ xbc, int ldx, const float* __restrict__ dtsrc, int lddt, int dt_col0,
+                const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
+                float* __restrict__ state, const int* __restrict__ seq_slots, float* __restrict__ y, int n_heads,
+                int head_dim, int n_state, int n_groups, int vec_rows) {
+    int p0 = blockIdx.x * SC_PT, head = blockIdx.y, b = blockIdx.z;
+    int tid = threadIdx.x, r = tid % SC_R, pl = tid / SC_R;
+    int group = head / (n_heads / n_groups);
+    int inner = n_heads * head_dim;
+    float* st_head = state + ((size_t)seq_slots[b] * n_heads + head) * head_dim * n_state;
+    const float* row = xbc + (size_t)b * ldx;
+    const float* brow = row + inner + (size_t)group * n_state;
+    const float* crow = brow + (size_t)n_groups * n_state;
+    float s[SC_PP][NI], bv[NI], cv[NI], xv[SC_PP];
+    // (B and C are read like a column of the state; their rows start on 16 bytes where the vector form is taken:
+    // the caller checks the strides)
+    sc_load_state<NI>(bv, brow, r, vec_rows ? n_state : -1, true);
+    sc_load_state<NI>(cv, crow, r, vec_rows ? n_state : -1, true);
+    if (!vec_rows) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             int n = r * NI + i;
-            if (p < head_dim && n < n_state) st_head[(size_t)p * n_state + n] = s[j][i];
+            bool ok = n < n_state;
+            bv[i] = ok ? brow[n] : 0.f;
+            cv[i] = ok ? crow[n] : 0.f;
         }
+    }
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+        sc_load_state<NI>(s[j], st_head + (size_t)min(p, head_dim - 1) * n_state, r, n_state, p < head_dim);
+    }
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+        xv[j] = p < head_dim ? row[(size_t)head * head_dim + p] : 0.f;
+    }
+    float dt = rc_softplus(dtsrc[(size_t)b * lddt + dt_col0 + head] + dt_bias[head]);
+    float dec = expf(-expf(a_log[head]) * dt), skip = d_skip[head];
+    float part[SC_PP];
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        float dtx = dt * xv[j], q = 0.f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            s[j][i] = fmaf(dec, s[j][i], dtx * bv[i]);
+            q = fmaf(s[j][i], cv[i], q);
+        }
+        part[j] = row16_sum(q);
+    }
+#pragma unroll
+    for (int j = 0; j < SC_PP; ++j) {
+        int p = p0 + pl * SC_PP + j;
+        if (p >= head_dim) continue;
+        if (r == 0) y[(size_t)b * inner + (size_t)head * head_dim + p] = fmaf(skip, xv[j], part[j]);
+        sc_store_state<NI>(s[j], st_head + (size_t)p * n_state, r, n_state, true);
     }
 }
 
@@ -399,6 +488,26 @@ ROCML_EXPORT int rocml_ssd_scan(const float* xbc, int ldx, const float* dtsrc, i
     dim3 grid(ceil_div(head_dim, SC_PT), n_heads, n_seqs);
     int ni = ceil_div(n_state, SC_R);
     ni = ni <= 4 ? ni : ni <= 6 ? 6 : ni <= 8 ? 8 : ni <= 12 ? 12 : 16;
+    if (n_tokens == n_seqs) {          // one token per sequence (every sequence of a step brings at least one)
+#define STEP(NI_)                                                                                              \
+    ssd_step_kernel<NI_><<<grid, RC_BLOCK, 0, stream>>>(xbc, ldx, dtsrc, lddt, dt_col0, dt_bias, a_log, d_skip, state, \
+                                                        seq_slots, y, n_heads, head_dim, n_state, n_groups, vec_rows)
+        // B and C rows as 16-byte pieces: every row and every group's part starts on a multiple of 4 numbers
+        int vec_rows = ldx % 4 == 0 && (n_heads * head_dim) % 4 == 0 && n_state % 4 == 0 && ((uintptr_t)xbc & 15) == 0;
+        switch (ni) {
+            case 1: STEP(1); break;
+            case 2: STEP(2); break;
+            case 3: STEP(3); break;
+            case 4: STEP(4); break;
+            case 6: STEP(6); break;
+            case 8: STEP(8); break;
+            case 12: STEP(12); break;
+            default: STEP(16); break;
+        }
+#undef STEP
+        ROCML_CHECK_LAUNCH("ssd_scan step");
+        return 0;
+    }
     int tc = ni <= 8 ? SC_MAX_TC : SC_MAX_TC / 2;          // 48 KB of LDS at most
     size_t lds = (size_t)(2 * tc * SC_R * ni + 2 * tc * SC_PT + 2 * tc) * sizeof(float);
     // whole 16-byte pieces: every row of x, B and C starts on a multiple of 4 numbers and ends on one
