@@ -58,13 +58,14 @@ CFG_A = config(211, 72, [
 
 # B: sizes the matrix-core kernels know: key heads of 64 and 128 with value heads of the same size, widths
 # that are multiples of 8 (the experts' products then run on the matrix cores in bfloat16), states of 64
-# and 128, more experts, a stretch that changes every 64 positions (inside the prompts).
+# and 128, more experts, a stretch that changes every 64 positions (inside the prompts).  Its attention
+# scales are twice 1/sqrt(dim), not eight times: it is the model that bfloat16 runs are judged on.
 CFG_B = config(300, 128, [
-    layer(left(4, 1, 64, 64, 0.5, (0.5, 64)), right(4, 32, 64, 2, 4, 2), dense(256, 1.5)),
-    layer(left(2, 2, 128, 128, 0.35, (0.4, 100)), right(2, 64, 128, 1, 4, 1), moe(8, 64, 3, (4, 2))),
-    layer(left(4, 2, 64, 64, 0.6), right(8, 16, 16, 4, 3, 8), moe(16, 32, 4, (2, 1))),
-    layer(left(8, 4, 32, 32, 0.7, (1.0, 7)), right(4, 32, 40, 4, 2, 4), dense(192, 4.0)),
-], alpha=3.0, scale=12.0)
+    layer(left(4, 1, 64, 64, 0.25, (0.45, 64)), right(4, 32, 64, 2, 4, 2), dense(224, 1.25)),
+    layer(left(2, 2, 128, 128, 0.18, (0.4, 100)), right(2, 64, 128, 1, 4, 1), moe(8, 64, 3, (4, 2))),
+    layer(left(4, 2, 64, 64, 0.3), right(8, 16, 16, 4, 3, 8), moe(16, 32, 4, (4, 3))),
+    layer(left(8, 4, 32, 32, 0.35, (1.0, 7)), right(4, 32, 40, 4, 2, 4), dense(192, 4.0)),
+], alpha=2.5, scale=9.0)
 
 # C: the values that make mechanisms vanish or coincide: one head everywhere, a convolution of one tap (no
 # inputs are kept), a state of one number, every expert chosen, all groups kept, a residual scale and an

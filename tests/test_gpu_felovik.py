@@ -23,10 +23,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TOL = {"float32": 3e-4}
 # bfloat16: these models are made to turn small differences into large ones (attention scales far above
 # 1/sqrt(dim), a single chosen expert, norms over parts of one value in C), so a rounding now and then flips
-# a choice and one position is off by its whole size: the 32-bit runs pin every position, the bfloat16 runs
-# pin most of them against the plain implementation and all of them against each other (a fault of the
-# cache, the state or the batch shows between two bfloat16 runs that should agree).
-BF16_MOST = {"A": (0.9, 6e-2), "B": (0.9, 6e-2), "C": (0.5, 1e-1)}
+# a choice of experts, and what that position then writes into the recurrence's state and the keys reaches every
+# later position of its sequence: the 32-bit runs pin every position, the bfloat16 runs pin the bulk of them
+# against the plain implementation (a median: a sequence may be off from its first flipped choice on) and against
+# each other (a fault of the cache, the state or the batch shows between two bfloat16 runs that should agree).
+BF16_MOST = {"A": (0.5, 4e-2), "B": (0.5, 4e-2), "C": (0.5, 1e-1)}
 # (A and C run the same kernels whatever the step's shape and agree to the last bit; B's head sizes take the
 # matrix-core attention, whose prompt and single-token kernels round differently)
 BF16_SAME = {"A": (0.98, 3e-2), "B": (0.9, 6e-2), "C": (0.98, 3e-2)}
