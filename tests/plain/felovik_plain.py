@@ -10,7 +10,6 @@ stored ``[out, in]``.  The arithmetic type is the type of the tensors handed in 
 """
 from __future__ import annotations
 
-import math
 from typing import Dict, List, Optional, Sequence
 
 import torch

@@ -4,7 +4,6 @@ made to stand out far away and at page borders (prompt and single-token kernels)
 the causal convolution and the recurrence carried through pieces, slots used again, decays close to
 one and to zero, the gated norm in parts, the limited gated activation, the experts' choice with and
 without groups, the experts' products on both kinds of kernel, and the sum with its norm."""
-import math
 
 import pytest
 import torch
